@@ -45,11 +45,14 @@ HIP_SOURCES = [
 #           residual, norms, gated units, routers)
 #   seq     masked softmax attention + decayed linear recurrences
 #   ssm     selective state-space scan + sigmoid attention
+#   hyper   multi-stream residual mixing, input convolutions, latent-attention
+#           row steps
 MIX_GROUPS = {
     "glue": (PKG_DIR / "libafglue.so", ["mix_glue.hip"]),
     "seq": (PKG_DIR / "libafmix.so", ["mix_seq.hip", "mix_attn_mfma.hip"]),
     "ssm": (PKG_DIR / "libafssm.so", ["mix_ssm.hip", "mix_sigattn.hip",
                                        "mix_sigattn_mfma.hip"]),
+    "hyper": (PKG_DIR / "libafhyper.so", ["mix_hyper.hip"]),
 }
 MIX_SOURCES = [s for _lib, srcs in MIX_GROUPS.values() for s in srcs]
 MIX_LIB = MIX_GROUPS["seq"][0]
@@ -64,7 +67,7 @@ def _needs_build(lib: Path = LIB, sources=None) -> bool:
         return True
     lib_m = lib.stat().st_mtime
     deps = [CSRC / s for s in (sources or HIP_SOURCES)] + \
-        [CSRC / "common.h", Path(__file__)]
+        [CSRC / "common.h", CSRC / "mix_attn.h", Path(__file__)]
     return any(d.stat().st_mtime > lib_m for d in deps)
 
 

@@ -18,6 +18,7 @@
 //   B: lane holds B[k = (lane>>4)*8 + j][n = lane&15]
 //   C: lane reg r holds C[m = (lane>>4)*4 + r][n = lane&15]
 #include "common.h"
+#include "mix_attn.h"
 
 namespace {
 
@@ -52,12 +53,13 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
     const i32* __restrict__ bt, const i32* __restrict__ cu,
     const i32* __restrict__ q_start, const i32* __restrict__ tile_seq,
     const i32* __restrict__ tile_q0, float scale, int H, int G, int dk, int dv,
-    int page, int maxp, int chunk, int window, i64 ldq) {
+    int page, int maxp, int chunk, int window, i64 ldq, AttnExtra ex) {
   constexpr int KS = DKC * 32 + 8;   // K row stride in LDS (elements)
   constexpr int VS = 72;             // V^T / P row stride (64 tokens + pad)
   __shared__ u16 k_lds[64 * KS];
   __shared__ u16 v_lds[DVT * 16 * VS];
   __shared__ u16 p_lds[4 * 16 * VS];
+  __shared__ float bias_lds[128];    // distance bias of this tile's distances
 
   const int tile = blockIdx.x, h = blockIdx.y;
   const int g = h / (H / G);
@@ -92,11 +94,15 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
   }
   float m[4], l[4];
   f32x4 o_acc[DVT];
+  // the sink enters as a key of score sink[h] and value 0 seen by every row
+  const float m0 = ex.sink ? ex.sink[h] : AF_NEG_INF;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) { m[r] = AF_NEG_INF; l[r] = 0.f; }
+  for (int r = 0; r < 4; ++r) { m[r] = m0; l[r] = ex.sink ? 1.f : 0.f; }
 #pragma unroll
   for (int dt = 0; dt < DVT; ++dt) o_acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   u16* pw = p_lds + wid * 16 * VS;
+  const float r1 = ex.r1 ? ex.r1[h] : 0.f, r2 = ex.r1 ? ex.r2[h] : 0.f;
+  const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
 
   for (int kv0 = lo; kv0 <= p_last; kv0 += 64) {
     __syncthreads();   // fragment reads of the previous tile are done
@@ -117,15 +123,21 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
       const int j0 = kv0 + tp * 2;
       s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
       if (j0 <= p_last)
-        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * dv, e0, dv);
+        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * ex.ldv, e0, dv);
       if (j0 + 1 <= p_last)
-        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * dv, e0, dv);
+        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * ex.ldv, e0, dv);
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
         const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
                                 ((uint32_t)(unsigned short)c8[jj] << 16);
         *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
       }
+    }
+    // distance bias for every distance between a row and a key of the tile:
+    // entry i is distance i + (p0 - kv0 - 63); keys ahead of a row are masked
+    if (ex.r1 && threadIdx.x < 127) {
+      const int dist = (int)threadIdx.x + p0 - kv0 - 63;
+      bias_lds[threadIdx.x] = dist > 0 ? attn_dist_bias(r1, r2, dist) : 0.f;
     }
     __syncthreads();
     // keys of this tile that any row of the wave may see
@@ -157,7 +169,10 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
         const int j = kv0 + st * 16 + (lane & 15);
-        sr[st] = (j <= p && j >= rlo) ? s_acc[st][r] * scale : AF_NEG_INF;
+        float sv = s_acc[st][r] * scale;
+        if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
+        if (ex.r1) sv -= bias_lds[(p - p0) - (j - kv0) + 63];
+        sr[st] = (j <= p && j >= rlo) ? sv : AF_NEG_INF;
         tmax = fmaxf(tmax, sr[st]);
       }
       tmax = group16_max_f32(tmax);
@@ -222,12 +237,20 @@ AF_EXPORT int afm_attn_prefill_mfma(
     void* out, const void* q, const void* kc, const void* vc, const void* bt,
     const void* cu, const void* q_start, const void* tile_seq,
     const void* tile_q0, float scale, int ntiles, int H, int G, int dk, int dv,
-    int page, int maxp, int chunk, int window, i64 ldq, void* stream) {
+    int page, int maxp, int chunk, int window, i64 ldq, const void* sink,
+    float cap, const void* r1, const void* r2, i64 ldv, void* stream) {
   if (ntiles == 0) return 0;
-  if (G <= 0 || H % G || dk < 1 || dv < 1 || dk > 128 || dv > 128) return 9003;
+  if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
+  if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
   const bool vec = (dk % 8 == 0) && (dv % 8 == 0) && (ldq % 8 == 0) &&
+                   (ldv % 8 == 0) &&
                    ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&
                    ((uintptr_t)vc % 16 == 0);
+  // wide heads exist in the 16-byte-aligned form only; 9004 sends the caller
+  // to the row kernel
+  if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
+  const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
+                     cap, ldv};
   dim3 grid(ntiles, H), blk(256);
   hipStream_t s = (hipStream_t)stream;
 #define APM(DKC, DVT, VEC)                                                     \
@@ -235,9 +258,11 @@ AF_EXPORT int afm_attn_prefill_mfma(
       (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,                \
       (const i32*)bt, (const i32*)cu, (const i32*)q_start,                     \
       (const i32*)tile_seq, (const i32*)tile_q0, scale, H, G, dk, dv, page,    \
-      maxp, chunk, window, ldq)
+      maxp, chunk, window, ldq, ex)
   const bool small = dk <= 64 && dv <= 64;
-  if (small && vec) APM(2, 4, true);
+  if (dk > 320 || dv > 256) APM(18, 32, true);
+  else if (dk > 128 || dv > 128) APM(10, 16, true);
+  else if (small && vec) APM(2, 4, true);
   else if (small) APM(2, 4, false);
   else if (vec) APM(4, 8, true);
   else APM(4, 8, false);

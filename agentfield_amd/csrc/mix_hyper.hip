@@ -1,0 +1,472 @@
+// Glue of hyper-connected decoders: several fp32 residual streams per token
+// mixed by small learned matrices, an RMSNorm and a short causal convolution
+// in front of every sublayer, and the row-wise steps of latent attention
+// (latent norm, interleaved rotary positions, cache append, query assembly,
+// gated head outputs).
+//
+// Storage dtype S is bf16 (raw u16) or fp32.  The streams, norm statistics,
+// convolution inputs and sums, angles and gates are fp32; S is what the
+// projections read and write.
+#include "common.h"
+
+namespace {
+
+template <typename S> __device__ __forceinline__ float ldf(const S* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename S> __device__ __forceinline__ void stf(S* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+// V consecutive elements as floats (V = 4: one 8- or 16-byte access)
+template <typename S, int V>
+__device__ __forceinline__ void ldv(const S* p, float (&o)[4]) {
+  if constexpr (V == 4) {
+    if constexpr (sizeof(S) == 2) {
+      const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = bf2f((u16)v[j]);
+    } else {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = v[j];
+    }
+  } else {
+    o[0] = ldf<S>(p);
+    o[1] = o[2] = o[3] = 0.f;
+  }
+}
+template <typename S, int V>
+__device__ __forceinline__ void stv(S* p, const float (&o)[4]) {
+  if constexpr (V == 4) {
+    if constexpr (sizeof(S) == 2) {
+      s16x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (short)f2bf(o[j]);
+      *reinterpret_cast<s16x4*>(p) = v;
+    } else {
+      *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+    }
+  } else {
+    stf<S>(p, o[0]);
+  }
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum_f32(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float s = red[0] + red[1] + red[2] + red[3];
+  __syncthreads();
+  return s;
+}
+
+// ------------------------------------------------------------ embedding
+// x[t, s, :] = table[ids[t]] for every stream s.
+template <typename S>
+__global__ void __launch_bounds__(256) embed_streams_kernel(
+    float* __restrict__ x, const S* __restrict__ table,
+    const i32* __restrict__ ids, int ns, int W) {
+  const int t = blockIdx.x;
+  const S* row = table + (size_t)ids[t] * W;
+  float* xr = x + (size_t)t * ns * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = ldf<S>(row + c);
+    for (int s = 0; s < ns; ++s) xr[(size_t)s * W + c] = v;
+  }
+}
+
+// ------------------------------------------------------------ stream step
+// One workgroup per token row.  With y: the streams take the sublayer output
+// in, all at once from the old ones:
+//     x_r <- sum_s mix[s, r] x_s + out[r] y            (r = 0..ns-1)
+// With in: the next sublayer's input is read out, u = sum_r in[r] x_r, and
+// left in `n` either as it is (norm_mode 0) or as u / rms(u) * (1 + w)
+// (norm_mode 1).  MS bounds the stream count; V columns per access.
+template <typename S, int MS, int V>
+__global__ void __launch_bounds__(256) hyper_step_kernel(
+    float* __restrict__ x, const S* __restrict__ y, i64 ldy,
+    const float* __restrict__ mixm, const float* __restrict__ outv,
+    const float* __restrict__ inv, const S* __restrict__ normw, float eps,
+    float* __restrict__ n, int ns, int W, int norm_mode) {
+  __shared__ float s_mix[MS * MS], s_in[MS], s_out[MS], red[4];
+  const int t = blockIdx.x;
+  if (threadIdx.x < MS * MS) {
+    const int s = threadIdx.x / MS, r = threadIdx.x % MS;
+    s_mix[threadIdx.x] = (y && s < ns && r < ns) ? mixm[s * ns + r] : 0.f;
+  }
+  if (threadIdx.x < MS) {
+    s_in[threadIdx.x] = (inv && (int)threadIdx.x < ns) ? inv[threadIdx.x] : 0.f;
+    s_out[threadIdx.x] = (y && (int)threadIdx.x < ns) ? outv[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  float* xr = x + (size_t)t * ns * W;
+  float* nr = n ? n + (size_t)t * W : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+    float xs[MS][4];
+#pragma unroll
+    for (int s = 0; s < MS; ++s)
+      if (s < ns) ldv<float, V>(xr + (size_t)s * W + c, xs[s]);
+    if (y) {
+      float yv[4], nw[MS][4];
+      ldv<S, V>(y + (size_t)t * ldy + c, yv);
+#pragma unroll
+      for (int r = 0; r < MS; ++r) {
+        if (r >= ns) continue;
+#pragma unroll
+        for (int j = 0; j < V; ++j) nw[r][j] = s_out[r] * yv[j];
+#pragma unroll
+        for (int s = 0; s < MS; ++s)
+          if (s < ns) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) nw[r][j] += s_mix[s * MS + r] * xs[s][j];
+          }
+      }
+#pragma unroll
+      for (int r = 0; r < MS; ++r)
+        if (r < ns) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) xs[r][j] = nw[r][j];
+          stv<float, V>(xr + (size_t)r * W + c, nw[r]);
+        }
+    }
+    if (inv) {
+      float u[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < MS; ++r)
+        if (r < ns) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) u[j] += s_in[r] * xs[r][j];
+        }
+#pragma unroll
+      for (int j = 0; j < V; ++j) ss += u[j] * u[j];
+      stv<float, V>(nr + c, u);
+    }
+  }
+  if (!inv || norm_mode == 0) return;
+  const float rinv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)W + eps);
+  // every thread rescales the columns it wrote itself
+  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+    float u[4], w4[4];
+    ldv<float, V>(nr + c, u);
+    ldv<S, V>(normw + c, w4);
+#pragma unroll
+    for (int j = 0; j < V; ++j) u[j] *= rinv * (1.0f + w4[j]);
+    stv<float, V>(nr + c, u);
+  }
+}
+
+// ------------------------------------------------- input convolution
+// h[t, c] = n[t, c] + sum_j w[c, j] n[t - (taps-1-j), c]: a causal depthwise
+// convolution added to its own input.  Rows before the chunk come from the
+// sequence's slot of `state` [slots, taps-1, W] fp32 (oldest first), rows
+// before position 0 are zero.  One workgroup per (row, 256 channels).
+template <typename S>
+__global__ void __launch_bounds__(256) canon_conv_kernel(
+    S* __restrict__ h, const float* __restrict__ n, const S* __restrict__ w,
+    const float* __restrict__ state, const i32* __restrict__ row_seq,
+    const i32* __restrict__ cu, const i32* __restrict__ q_start,
+    const i32* __restrict__ sslot, int W, int taps) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int b = row_seq[t];
+  const int r = t - cu[b];
+  const int p = q_start[b] + r;
+  const int hist = taps - 1;
+  const float* st = state + (size_t)sslot[b] * (hist > 0 ? hist : 1) * W;
+  const float cur = n[(size_t)t * W + c];
+  float acc = cur;
+  for (int j = 0; j < taps; ++j) {
+    const int k = hist - j;                  // rows back
+    float v = 0.f;
+    if (k == 0) v = cur;
+    else if (p - k < 0) v = 0.f;
+    else if (r - k >= 0) v = n[(size_t)(t - k) * W + c];
+    else v = st[(size_t)(hist + r - k) * W + c];
+    acc += ldf<S>(w + (size_t)c * taps + j) * v;
+  }
+  stf<S>(h + (size_t)t * W + c, acc);
+}
+
+// After the convolution: the slot keeps the sequence's last taps-1 inputs.
+// A chunk shorter than that keeps the tail of the old content in front.
+__global__ void __launch_bounds__(256) canon_state_kernel(
+    float* __restrict__ state, const float* __restrict__ n,
+    const i32* __restrict__ cu, const i32* __restrict__ q_start,
+    const i32* __restrict__ sslot, int W, int taps) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int r0 = cu[b], len = cu[b + 1] - r0;
+  const int hist = taps - 1;
+  if (c >= W || len <= 0 || hist <= 0) return;
+  float* st = state + (size_t)sslot[b] * hist * W;
+  const int qs = q_start[b];
+  for (int i = 0; i < hist; ++i) {
+    const int rr = len - hist + i;           // chunk row kept in place i
+    float v;
+    if (qs + rr < 0) v = 0.f;
+    else if (rr >= 0) v = n[(size_t)(r0 + rr) * W + c];
+    else v = st[(size_t)(hist + rr) * W + c];     // = old place len + i > i
+    st[(size_t)i * W + c] = v;
+  }
+}
+
+// ------------------------------------------------------- latent attention
+// One workgroup per row.  The down projection's row holds the latent (first
+// R values) and one rotary key part (rd values); the latent is RMS-normed
+// with a plain weight, the key part rotated, and [latent | key part] goes to
+// the key pages [P, 1, page, R + rd] at `slot`.  The query of head h is put
+// together as [qa[h, t, :R] | rotate(q[t, h, dim:dim+rd])]: qa is the
+// unrotated query already multiplied into latent space.  Rotation pairs
+// element 2i with 2i+1 for i < rot/2, angle = position * inv_freq[i] in fp32.
+template <typename S>
+__global__ void __launch_bounds__(256) latent_prep_kernel(
+    S* __restrict__ qf, S* __restrict__ kc, const S* __restrict__ q, i64 ldq,
+    const S* __restrict__ dkv, i64 lddkv, const S* __restrict__ qa,
+    const S* __restrict__ normw, const float* __restrict__ inv_freq,
+    const i32* __restrict__ positions, const i64* __restrict__ slots,
+    float eps, int T, int H, int dim, int rd, int R, int rot) {
+  __shared__ float red[4];
+  extern __shared__ float cs[];              // [rot/2] cos, [rot/2] sin
+  const int t = blockIdx.x;
+  const int half = rot / 2;
+  const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < half; i += 256) {
+    float sn, c;
+    sincosf(pos * inv_freq[i], &sn, &c);
+    cs[i] = c;
+    cs[half + i] = sn;
+  }
+  const S* dr = dkv + (size_t)t * lddkv;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < R; i += 256) {
+    const float v = ldf<S>(dr + i);
+    ss += v * v;
+  }
+  const float rinv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)R + eps);
+  const i64 sl = slots[t];
+  const int dkc = R + rd;
+  if (sl >= 0) {
+    S* kr = kc + (size_t)sl * dkc;           // one K/V head: slot * row
+    for (int i = threadIdx.x; i < R; i += 256)
+      stf<S>(kr + i, ldf<S>(dr + i) * rinv * ldf<S>(normw + i));
+    for (int i = threadIdx.x; i < rd; i += 256) {
+      float v = ldf<S>(dr + R + i);
+      if (i < rot) {
+        const int pr = i >> 1;
+        const float o = ldf<S>(dr + R + (i ^ 1));
+        v = (i & 1) ? v * cs[pr] + o * cs[half + pr]
+                    : v * cs[pr] - o * cs[half + pr];
+      }
+      stf<S>(kr + R + i, v);
+    }
+  }
+  const int dq = dim + rd;
+  for (int i = threadIdx.x; i < H * dkc; i += 256) {
+    const int h = i / dkc, e = i % dkc;
+    float v;
+    if (e < R) {
+      v = ldf<S>(qa + ((size_t)h * T + t) * R + e);
+    } else {
+      const int k = e - R;
+      const S* qr = q + (size_t)t * ldq + (size_t)h * dq + dim;
+      v = ldf<S>(qr + k);
+      if (k < rot) {
+        const int pr = k >> 1;
+        const float o = ldf<S>(qr + (k ^ 1));
+        v = (k & 1) ? v * cs[pr] + o * cs[half + pr]
+                    : v * cs[pr] - o * cs[half + pr];
+      }
+    }
+    stf<S>(qf + (size_t)t * H * dkc + i, v);
+  }
+}
+
+// out[t, h*dv + d] = o[h, t, d] * sigmoid(g[t, h*dv + d]): head-major
+// per-head results back to token rows, times the output gate.
+template <typename S>
+__global__ void __launch_bounds__(256) gate_heads_kernel(
+    S* __restrict__ out, const S* __restrict__ o, const S* __restrict__ g,
+    i64 ldg, int T, int H, int dv) {
+  const i64 total = (i64)T * H * dv;
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (i64)gridDim.x * 256) {
+    const int d = (int)(i % dv);
+    const int h = (int)((i / dv) % H);
+    const i64 t = i / ((i64)dv * H);
+    const float gv = ldf<S>(g + t * ldg + (i64)h * dv + d);
+    const float ov = ldf<S>(o + ((i64)h * T + t) * dv + d);
+    stf<S>(out + i, ov / (1.0f + expf(-gv)));
+  }
+}
+
+// out = max(z, 0)^2, rows of z at stride ldz.
+template <typename S, int V>
+__global__ void __launch_bounds__(256) relu2_kernel(
+    S* __restrict__ out, const S* __restrict__ z, i64 ldz, int T, int F) {
+  const i64 per = F / V;
+  const i64 total = (i64)T * per;
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (i64)gridDim.x * 256) {
+    const i64 t = i / per;
+    const int c = (int)(i % per) * V;
+    float v[4];
+    ldv<S, V>(z + t * ldz + c, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float r = fmaxf(v[j], 0.f);
+      v[j] = r * r;
+    }
+    stv<S, V>(out + t * F + c, v);
+  }
+}
+
+inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+AF_EXPORT int afm_embed_streams(void* x, const void* table, const void* ids,
+                                int T, int ns, int W, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (ns < 1) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    embed_streams_kernel<u16><<<T, 256, 0, s>>>((float*)x, (const u16*)table,
+                                                (const i32*)ids, ns, W);
+  else if (dt == 1)
+    embed_streams_kernel<float><<<T, 256, 0, s>>>(
+        (float*)x, (const float*)table, (const i32*)ids, ns, W);
+  else
+    return 9002;
+  return af_last_err();
+}
+
+template <typename S>
+static int launch_hyper_step(float* x, const void* y, i64 ldy,
+                             const float* mixm, const float* outv,
+                             const float* inv, const void* normw, float eps,
+                             float* n, int T, int ns, int W, int norm_mode,
+                             hipStream_t s) {
+  const bool vec = W % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(n) &&
+                   al16(y) && al16(normw);
+#define HS(MS, V)                                                            \
+  hyper_step_kernel<S, MS, V><<<T, 256, 0, s>>>(                             \
+      x, (const S*)y, ldy, mixm, outv, inv, (const S*)normw, eps, n, ns, W,  \
+      norm_mode)
+  if (ns <= 4) { if (vec) HS(4, 4); else HS(4, 1); }
+  else if (ns <= 8) { if (vec) HS(8, 4); else HS(8, 1); }
+  else { if (vec) HS(16, 4); else HS(16, 1); }
+#undef HS
+  return af_last_err();
+}
+
+// x [T, ns, W] fp32 in place; y [T, W] at row stride ldy (or null); mixm
+// [ns, ns] indexed [from, to], outv / inv [ns] fp32; normw [W]; n [T, W] fp32.
+AF_EXPORT int afm_hyper_step(void* x, const void* y, i64 ldy, const void* mixm,
+                             const void* outv, const void* inv,
+                             const void* normw, float eps, void* n, int T,
+                             int ns, int W, int norm_mode, int dt,
+                             void* stream) {
+  if (T == 0) return 0;
+  if (ns < 1 || ns > 16) return 9003;
+  if (y && (!mixm || !outv)) return 9003;
+  if (inv && (!n || (norm_mode == 1 && !normw))) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    return launch_hyper_step<u16>((float*)x, y, ldy, (const float*)mixm,
+        (const float*)outv, (const float*)inv, normw, eps, (float*)n, T, ns, W,
+        norm_mode, s);
+  if (dt == 1)
+    return launch_hyper_step<float>((float*)x, y, ldy, (const float*)mixm,
+        (const float*)outv, (const float*)inv, normw, eps, (float*)n, T, ns, W,
+        norm_mode, s);
+  return 9002;
+}
+
+// h [T, W] in the storage dtype; n [T, W] fp32; w [W, taps]; state [slots,
+// max(taps-1, 1), W] fp32.  Runs the convolution, then moves the slots on.
+AF_EXPORT int afm_canon_conv(void* h, const void* n, const void* w,
+                             void* state, const void* row_seq, const void* cu,
+                             const void* q_start, const void* sslot, int T,
+                             int B, int W, int taps, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (taps < 1) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(T, (W + 255) / 256);
+  if (dt == 0)
+    canon_conv_kernel<u16><<<grid, 256, 0, s>>>(
+        (u16*)h, (const float*)n, (const u16*)w, (const float*)state,
+        (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
+        (const i32*)sslot, W, taps);
+  else if (dt == 1)
+    canon_conv_kernel<float><<<grid, 256, 0, s>>>(
+        (float*)h, (const float*)n, (const float*)w, (const float*)state,
+        (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
+        (const i32*)sslot, W, taps);
+  else
+    return 9002;
+  if (taps > 1)
+    canon_state_kernel<<<dim3(B, (W + 255) / 256), 256, 0, s>>>(
+        (float*)state, (const float*)n, (const i32*)cu, (const i32*)q_start,
+        (const i32*)sslot, W, taps);
+  return af_last_err();
+}
+
+AF_EXPORT int afm_latent_prep(void* qf, void* kc, const void* q, i64 ldq,
+                              const void* dkv, i64 lddkv, const void* qa,
+                              const void* normw, const void* inv_freq,
+                              const void* positions, const void* slots,
+                              float eps, int T, int H, int dim, int rd, int R,
+                              int rot, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (rot < 0 || rot > rd || (rot & 1) || (rot && !inv_freq)) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t sm = (size_t)(rot > 0 ? rot : 1) * sizeof(float);
+  if (dt == 0)
+    latent_prep_kernel<u16><<<T, 256, sm, s>>>(
+        (u16*)qf, (u16*)kc, (const u16*)q, ldq, (const u16*)dkv, lddkv,
+        (const u16*)qa, (const u16*)normw, (const float*)inv_freq,
+        (const i32*)positions, (const i64*)slots, eps, T, H, dim, rd, R, rot);
+  else if (dt == 1)
+    latent_prep_kernel<float><<<T, 256, sm, s>>>(
+        (float*)qf, (float*)kc, (const float*)q, ldq, (const float*)dkv, lddkv,
+        (const float*)qa, (const float*)normw, (const float*)inv_freq,
+        (const i32*)positions, (const i64*)slots, eps, T, H, dim, rd, R, rot);
+  else
+    return 9002;
+  return af_last_err();
+}
+
+AF_EXPORT int afm_gate_heads(void* out, const void* o, const void* g, i64 ldg,
+                             int T, int H, int dv, int dt, void* stream) {
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const i64 total = (i64)T * H * dv;
+  const int grid = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  if (dt == 0)
+    gate_heads_kernel<u16><<<grid, 256, 0, s>>>((u16*)out, (const u16*)o,
+                                                (const u16*)g, ldg, T, H, dv);
+  else if (dt == 1)
+    gate_heads_kernel<float><<<grid, 256, 0, s>>>(
+        (float*)out, (const float*)o, (const float*)g, ldg, T, H, dv);
+  else
+    return 9002;
+  return af_last_err();
+}
+
+AF_EXPORT int afm_relu2(void* out, const void* z, i64 ldz, int T, int F,
+                        int dt, void* stream) {
+  if (T == 0 || F == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bool vec = F % 4 == 0 && ldz % 4 == 0 && al16(out) && al16(z);
+  const i64 total = (i64)T * (vec ? F / 4 : F);
+  const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+#define R2(S, V) relu2_kernel<S, V><<<grid, 256, 0, s>>>((S*)out, (const S*)z, ldz, T, F)
+  if (dt == 0) { if (vec) R2(u16, 4); else R2(u16, 1); }
+  else if (dt == 1) { if (vec) R2(float, 4); else R2(float, 1); }
+  else return 9002;
+#undef R2
+  return af_last_err();
+}

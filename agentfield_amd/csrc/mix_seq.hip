@@ -6,6 +6,7 @@
 // Storage dtype S is bf16 (raw u16) or fp32; scores, softmax, decays and the
 // recurrent state are fp32.
 #include "common.h"
+#include "mix_attn.h"
 
 namespace {
 
@@ -127,7 +128,7 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
     const S* __restrict__ vc, const i32* __restrict__ bt,
     const i32* __restrict__ row_seq, const i32* __restrict__ positions,
     float scale, int n_rh, int H, int G, int dk, int dv, int page, int maxp,
-    int chunk, int window, i64 ldq) {
+    int chunk, int window, i64 ldq, AttnExtra ex) {
   extern __shared__ float smem[];           // [4][dk + 64]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int rh = blockIdx.x * 4 + wave;
@@ -144,6 +145,8 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
   const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
   for (int d = lane; d < dk; d += 64) qs[d] = ldf<S>(qr + d) * scale;
   float m = AF_NEG_INF, l = 0.f;
+  if (ex.sink) { m = ex.sink[h]; l = 1.f; }
+  const float r1 = ex.r1 ? ex.r1[h] : 0.f, r2 = ex.r1 ? ex.r2[h] : 0.f;
   float acc[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
@@ -155,10 +158,11 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
       const S* kr = kc + (((size_t)pg * G + g) * page + (j % page)) * dk;
       float d0 = 0.f;
       for (int d = 0; d < dk; ++d) d0 += qs[d] * ldf<S>(kr + d);
-      s = d0;
+      s = attn_softcap(d0, ex.cap);
+      if (ex.r1) s -= attn_dist_bias(r1, r2, pos - j);
     }
     const float mn = fmaxf(m, wave_max_f32(s));
-    const float corr = expf(m - mn);
+    const float corr = (m <= AF_NEG_INF) ? 0.f : expf(m - mn);
     const float p = (j <= pos) ? expf(s - mn) : 0.f;
     l = l * corr + wave_sum_f32(p);
     m = mn;
@@ -174,7 +178,7 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
         for (int jj = 0; jj < cnt; ++jj) {
           const int jk = j0 + jj;
           const int pg = btr[jk / page];
-          a += ps[jj] * ldf<S>(vc + (((size_t)pg * G + g) * page + (jk % page)) * dv + d);
+          a += ps[jj] * ldf<S>(vc + (((size_t)pg * G + g) * page + (jk % page)) * ex.ldv + d);
         }
       }
       acc[i] = a;
@@ -233,7 +237,7 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
     const i32* __restrict__ row_seq, const i32* __restrict__ positions,
     float scale, int H, int G, int dk, int dv, int page, int maxp, int chunk,
     int window, i64 ldq, int lpk_log2, int lpv_log2, int kt, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, AttnExtra ex) {
   // nsplit > 1: the visible keys are cut into nsplit ranges, one workgroup
   // each (grid.z = head blocks x nsplit); unnormalised outputs and (max,
   // sum) go to part_o [T, H, nsplit, dv] / part_ml [T, H, nsplit, 2] and
@@ -246,8 +250,10 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
   float* m_run = red + 4 * GQ * dvp;           // [8]
   float* l_run = m_run + 8;                    // [8]
   float* corr = l_run + 8;                     // [8]
+  float* r1s = corr + 8;                       // [8] distance-bias factors
+  float* r2s = r1s + 8;                        // [8]
   const int dkp = (dk + EPL - 1) / EPL * EPL;
-  float* qs = corr + 8;                        // [GQ][dkp] scaled queries
+  float* qs = r2s + 8;                         // [GQ][dkp] scaled queries
   const int t = blockIdx.x, g = blockIdx.y;
   const int hpg = H / G;
   const int zh = blockIdx.z / nsplit, sp = blockIdx.z % nsplit;
@@ -255,6 +261,7 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
   const int nh = min(GQ, hpg - zh * GQ);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   int pos = positions[t];
+  const int qpos = pos;
   const i32* btr = bt + (size_t)row_seq[t] * maxp;
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
@@ -278,7 +285,15 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
   for (int gg = 0; gg < GQ; ++gg)
 #pragma unroll
     for (int j = 0; j < EPL; ++j) acc[gg][j] = 0.f;
-  if (threadIdx.x < GQ) { m_run[threadIdx.x] = AF_NEG_INF; l_run[threadIdx.x] = 0.f; }
+  if (threadIdx.x < GQ) {
+    // the sink joins the first key range only
+    const bool sk = ex.sink && sp == 0 && (int)threadIdx.x < nh;
+    m_run[threadIdx.x] = sk ? ex.sink[h0 + threadIdx.x] : AF_NEG_INF;
+    l_run[threadIdx.x] = sk ? 1.f : 0.f;
+    const bool rb = ex.r1 && (int)threadIdx.x < nh;
+    r1s[threadIdx.x] = rb ? ex.r1[h0 + threadIdx.x] : 0.f;
+    r2s[threadIdx.x] = rb ? ex.r2[h0 + threadIdx.x] : 0.f;
+  }
 
   for (int tile0 = lo; tile0 <= pos; tile0 += kt) {
     const int nk = min(kt, pos + 1 - tile0);
@@ -301,7 +316,11 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
       }
 #pragma unroll
       for (int gg = 0; gg < GQ; ++gg)
-        if (gg < nh) sc[gg * kt + kidx] = sco[gg];
+        if (gg < nh) {
+          float sv = attn_softcap(sco[gg], ex.cap);
+          if (ex.r1) sv -= attn_dist_bias(r1s[gg], r2s[gg], qpos - j);
+          sc[gg * kt + kidx] = sv;
+        }
     }
     __syncthreads();
     // ---- B: softmax statistics, wave w takes heads w, w+4, ... ----
@@ -341,7 +360,7 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int j = tile0 + min(kb + u * 4 * kpv + kiv, nk - 1);
-        const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dv;
+        const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * ex.ldv;
         load_slice<S, VEC>(vr, liv * EPL, dv, vv[u]);
       }
 #pragma unroll
@@ -643,7 +662,8 @@ static int launch_attention(void* out, const void* q, const void* kc,
                             const void* positions, float scale, int T, int H,
                             int G, int dk, int dv, int page, int maxp,
                             int chunk, int window, i64 ldq, int nsplit,
-                            float* part_o, float* part_ml, hipStream_t s) {
+                            float* part_o, float* part_ml, AttnExtra ex,
+                            hipStream_t s) {
   constexpr int EPL = 16 / (int)sizeof(S);
   if (dk <= 64 * EPL && dv <= 64 * EPL) {
     auto clog2 = [](int n) { int l = 0; while ((1 << l) < n) ++l; return l; };
@@ -653,9 +673,9 @@ static int launch_attention(void* out, const void* q, const void* kc,
     const int dvp = EPL << lpv;
     const int kt = dvp <= 128 ? 1024 : 512;
     const int dkp = (dk + EPL - 1) / EPL * EPL;
-    const size_t sm = ((size_t)gq * kt + 4 * gq * dvp + 24 +
+    const size_t sm = ((size_t)gq * kt + 4 * gq * dvp + 40 +
                        (size_t)gq * dkp) * sizeof(float);
-    const bool vec = dk % EPL == 0 && dv % EPL == 0 &&
+    const bool vec = dk % EPL == 0 && dv % EPL == 0 && ex.ldv % EPL == 0 &&
                      (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0;
     if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
     dim3 grid(T, G, ((hpg + gq - 1) / gq) * nsplit);
@@ -663,7 +683,7 @@ static int launch_attention(void* out, const void* q, const void* kc,
   attn_rows_kernel<S, GQ, VEC><<<grid, 256, sm, s>>>(                         \
       (S*)out, (const S*)q, (const S*)kc, (const S*)vc, (const i32*)bt,       \
       (const i32*)row_seq, (const i32*)positions, scale, H, G, dk, dv, page,  \
-      maxp, chunk, window, ldq, lpk, lpv, kt, nsplit, part_o, part_ml)
+      maxp, chunk, window, ldq, lpk, lpv, kt, nsplit, part_o, part_ml, ex)
     if (vec) {
       if (gq == 1) ROWS(1, true); else if (gq == 2) ROWS(2, true);
       else if (gq == 4) ROWS(4, true); else ROWS(8, true);
@@ -685,10 +705,11 @@ static int launch_attention(void* out, const void* q, const void* kc,
   masked_attention_kernel<S, MV><<<grid, 256, sm, s>>>(                      \
       (S*)out, (const S*)q, (const S*)kc, (const S*)vc, (const i32*)bt,      \
       (const i32*)row_seq, (const i32*)positions, scale, n_rh, H, G, dk, dv, \
-      page, maxp, chunk, window, ldq)
+      page, maxp, chunk, window, ldq, ex)
   if (dv <= 64) ATT(1);
   else if (dv <= 128) ATT(2);
-  else ATT(4);
+  else if (dv <= 256) ATT(4);
+  else ATT(8);
 #undef ATT
   return af_last_err();
 }
@@ -697,20 +718,24 @@ AF_EXPORT int afm_masked_attention(
     void* out, const void* q, const void* kc, const void* vc, const void* bt,
     const void* row_seq, const void* positions, float scale, int T, int H,
     int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
-    int nsplit, void* part_o, void* part_ml, int dt, void* stream) {
+    int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
+    const void* r1, const void* r2, i64 ldv, int dt, void* stream) {
   if (T == 0) return 0;
-  if (G <= 0 || H % G || dv > 256 || dk > 1024) return 9003;
+  if (G <= 0 || H % G || dv > 512 || dk > 1024) return 9003;
+  if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
+  const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
+                     cap, ldv};
   hipStream_t s = (hipStream_t)stream;
   if (dt == 0)
     return launch_attention<u16>(out, q, kc, vc, bt, row_seq, positions, scale,
                                  T, H, G, dk, dv, page, maxp, chunk, window,
                                  ldq, nsplit, (float*)part_o, (float*)part_ml,
-                                 s);
+                                 ex, s);
   if (dt == 1)
     return launch_attention<float>(out, q, kc, vc, bt, row_seq, positions,
                                    scale, T, H, G, dk, dv, page, maxp, chunk,
                                    window, ldq, nsplit, (float*)part_o,
-                                   (float*)part_ml, s);
+                                   (float*)part_ml, ex, s);
   return 9002;
 }
 

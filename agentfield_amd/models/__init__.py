@@ -1,6 +1,7 @@
 from .llama import LlamaConfig, LlamaForCausalLM, CONFIGS as _LLAMA_CONFIGS
 from .hybrid import HYBRID_CONFIGS, ReperaxConfig, ReperaxForCausalLM
 from .zudisun import ZUDISUN_CONFIGS, ZudisunConfig, ZudisunForCausalLM
+from .fugevik import FUGEVIK_CONFIGS, FugevikConfig, FugevikForCausalLM
 from .registry import (architecture_of, build_model, load_model,
                        register_architecture)
 
@@ -8,8 +9,10 @@ from .registry import (architecture_of, build_model, load_model,
 CONFIGS = dict(_LLAMA_CONFIGS)
 CONFIGS.update(HYBRID_CONFIGS)
 CONFIGS.update(ZUDISUN_CONFIGS)
+CONFIGS.update(FUGEVIK_CONFIGS)
 
 __all__ = ["LlamaConfig", "LlamaForCausalLM", "ReperaxConfig",
            "ReperaxForCausalLM", "ZudisunConfig",
-           "ZudisunForCausalLM", "CONFIGS", "architecture_of", "build_model",
+           "ZudisunForCausalLM", "FugevikConfig", "FugevikForCausalLM",
+           "CONFIGS", "architecture_of", "build_model",
            "load_model", "register_architecture"]

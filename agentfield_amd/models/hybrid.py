@@ -219,7 +219,8 @@ class HybridCache:
     one entry per layer run (a looped layer counts once per pass) with
 
       "kv":    (kv_heads, dk, dv) or None - K/V pages [P, G, page, dk] /
-               [P, G, page, dv] in the model dtype
+               [P, G, page, dv] in the model dtype (dv 0: key pages only,
+               for layers whose values are part of the key rows)
       "state": {name: (shape, "f32" | "model")} - per-sequence tensors
                [slots, *shape] (recurrent matrices, token-shift rows,
                convolution inputs, ...)
@@ -242,8 +243,9 @@ class HybridCache:
                 G, dk, dv = kv
                 self.k[r] = torch.zeros(num_pages, G, page_size, dk,
                                         dtype=dtype, device=device)
-                self.v[r] = torch.zeros(num_pages, G, page_size, dv,
-                                        dtype=dtype, device=device)
+                if dv > 0:
+                    self.v[r] = torch.zeros(num_pages, G, page_size, dv,
+                                            dtype=dtype, device=device)
             for name, (shape, kind) in (need.get("state") or {}).items():
                 self.state.setdefault(name, {})[r] = torch.zeros(
                     num_slots, *shape, device=device,

@@ -148,9 +148,10 @@ def _mix_sigs() -> dict:
             "afm_qk_norm_cache": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i,
                                   i, i, i, i64, i64, i64, i, p],
             "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i,
-                                     i, i, i, i64, i, p, p, i, p],
+                                     i, i, i, i64, i, p, p, p, f, p, p, i64,
+                                     i, p],
             "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i,
-                                      i, i, i, i, i, i64, p],
+                                      i, i, i, i, i, i64, p, f, p, p, i64, p],
             "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
                                 i, i, i, i, i, i64, i64, i64, i64, i, p],
         },
@@ -167,6 +168,15 @@ def _mix_sigs() -> dict:
             "afm_sigmoid_attention": [p, p, p, p, p, p, p, p, p, p, i, i, p, p,
                                       p, i64, f, i, i, i, i, i, i, i, i, i, i,
                                       p],
+        },
+        "hyper": {
+            "afm_embed_streams": [p, p, p, i, i, i, i, p],
+            "afm_hyper_step": [p, p, i64, p, p, p, p, f, p, i, i, i, i, i, p],
+            "afm_canon_conv": [p, p, p, p, p, p, p, p, i, i, i, i, i, p],
+            "afm_latent_prep": [p, p, p, i64, p, i64, p, p, p, p, p, f, i, i,
+                                i, i, i, i, i, p],
+            "afm_gate_heads": [p, p, p, i64, i, i, i, i, p],
+            "afm_relu2": [p, p, i64, i, i, i, p],
         },
     }
 

@@ -204,17 +204,32 @@ def qk_norm_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
 
 def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
-                     vcache: torch.Tensor, md, positions: torch.Tensor,
+                     vcache: torch.Tensor | None, md, positions: torch.Tensor,
                      scale: float, heads: int, chunk: int = 0,
-                     window: int = 0) -> torch.Tensor:
+                     window: int = 0, sink: torch.Tensor | None = None,
+                     softcap: float = 0.0,
+                     log_bias: tuple | None = None,
+                     v_width: int = 0) -> torch.Tensor:
     """Softmax attention of packed rows over the paged cache.  Row at
     position i sees key j iff j <= i, and (chunk > 0) floor(j/chunk) ==
     floor(i/chunk), and (window > 0) j > i - window.  Positions are absolute
-    in the sequence.  q [T, H*dk] -> [T, H*dv]; scores and softmax in fp32."""
+    in the sequence.  q [T, H*dk] -> [T, H*dv]; scores and softmax in fp32.
+
+    Optional terms, per head h: s = q.k * scale; softcap > 0: s <- softcap *
+    tanh(s / softcap); log_bias (r1, r2) [H] fp32 each: s <- s - r1[h] *
+    ln(1 + r2[h] * (i - j)); sink [H] fp32: exp(sink[h]) joins the softmax
+    denominator (a term without key or value, not scaled).  vcache None: the
+    values are the first v_width elements of the key rows."""
     T = q.shape[0]
     _, G, page, dk = kcache.shape
-    dv = vcache.shape[3]
+    if vcache is None:
+        if not 0 < v_width <= dk:
+            raise ValueError("values inside the key rows need 0 < v_width <= dk")
+        dv, ldv, vsrc = v_width, dk, kcache
+    else:
+        dv, ldv, vsrc = vcache.shape[3], vcache.shape[3], vcache
     H = heads
+    r1, r2 = log_bias if log_bias is not None else (None, None)
     if not _gpu(q):
         out = torch.zeros(T, H, dv, dtype=torch.float32)
         qf = q.float().view(T, H, dk)
@@ -231,16 +246,26 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             js = torch.arange(lo, i + 1)
             pg = bt[rs[t]][js // page]
             kk = kcache[pg, :, js % page].float()      # [n, G, dk]
-            vv = vcache[pg, :, js % page].float()
+            vv = vsrc[pg, :, js % page][..., :dv].float()
             kk = kk.repeat_interleave(H // G, dim=1)
             vv = vv.repeat_interleave(H // G, dim=1)
             s = torch.einsum("nhd,hd->hn", kk, qf[t]) * scale
-            out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            if r1 is not None:
+                s = s - r1.float()[:, None] * torch.log(
+                    1.0 + r2.float()[:, None] * (i - js).float()[None])
+            if sink is not None:
+                s = torch.cat([s, sink.float()[:, None]], 1)
+            w = torch.softmax(s, -1)[:, :js.numel()]
+            out[t] = torch.einsum("hn,nhd->hd", w, vv)
         return out.view(T, H * dv).to(q.dtype)
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     lens = getattr(md, "seq_lens", None)
-    if (q.dtype == torch.bfloat16 and lens is not None and dk <= 128
-            and dv <= 128 and max(lens) >= MFMA_MIN_ROWS):
+    extra = (_lib.ptr(sink), float(softcap), _lib.ptr(r1), _lib.ptr(r2),
+             int(ldv))
+    if (q.dtype == torch.bfloat16 and lens is not None and dk <= 576
+            and dv <= 512 and max(lens) >= MFMA_MIN_ROWS):
         # prompt portions: 64-row tiles on the matrix cores
         ts, tq = [], []
         for b, ln in enumerate(lens):
@@ -250,14 +275,15 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
         tile_seq = torch.tensor(ts, dtype=torch.int32, device=q.device)
         tile_q0 = torch.tensor(tq, dtype=torch.int32, device=q.device)
         rc = _L().afm_attn_prefill_mfma(
-            _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
+            _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vsrc),
             _lib.ptr(md.block_table), _lib.ptr(md.cu_seqlens),
             _lib.ptr(md.q_start), _lib.ptr(tile_seq), _lib.ptr(tile_q0),
             float(scale), len(ts), H, G, dk, dv, page,
             md.block_table.shape[1], int(chunk), int(window), _rowstride(q),
-            _lib.cur_stream())
-        _lib.check(rc, "afm_attn_prefill_mfma")
-        return out
+            *extra, _lib.cur_stream())
+        if rc != 9004:          # 9004: no tile kernel for this head geometry
+            _lib.check(rc, "afm_attn_prefill_mfma")
+            return out
     # few rows and many visible keys: cut the keys over several workgroups
     # (about 2048 in flight) and merge the partial softmaxes
     reach = min(x for x in (chunk, window, md.block_table.shape[1] * page)
@@ -272,11 +298,11 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
         part_ml = torch.empty(T, H, nsplit, 2, dtype=torch.float32,
                               device=q.device)
     rc = _L().afm_masked_attention(
-        _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
+        _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vsrc),
         _lib.ptr(md.block_table), _lib.ptr(md.row_seq), _lib.ptr(positions),
         float(scale), T, H, G, dk, dv, page, md.block_table.shape[1],
         int(chunk), int(window), _rowstride(q), nsplit, _lib.ptr(part_o),
-        _lib.ptr(part_ml), _code(q), _lib.cur_stream())
+        _lib.ptr(part_ml), *extra, _code(q), _lib.cur_stream())
     _lib.check(rc, "afm_masked_attention")
     return out
 
@@ -878,4 +904,190 @@ def sigmoid_attention(q: torch.Tensor, kcache: torch.Tensor,
         dk, dv, page, md.block_table.shape[1], nsplit, int(window), _code(q),
         _lib.cur_stream())
     _lib.check(rc, "afm_sigmoid_attention")
+    return out
+
+
+# =====================================================================
+# Ops of hyper-connected decoders: several fp32 residual streams per token
+# mixed by learned matrices, a norm and a short causal convolution in front
+# of every sublayer, latent attention (one normed latent + one rotary key
+# part per token in the pages), squared-ReLU feed-forward.
+# =====================================================================
+def embed_streams(ids: torch.Tensor, table: torch.Tensor,
+                  streams: int) -> torch.Tensor:
+    """x[t, s] = table[ids[t]] for every stream s: fp32 [T, streams, W]."""
+    T, W = ids.numel(), table.shape[1]
+    if not _gpu(table):
+        return table[ids.long()].float()[:, None, :].repeat(1, streams, 1)
+    x = torch.empty(T, streams, W, dtype=torch.float32, device=table.device)
+    rc = _L().afm_embed_streams(_lib.ptr(x), _lib.ptr(table), _lib.ptr(ids), T,
+                                streams, W, _code(table), _lib.cur_stream())
+    _lib.check(rc, "afm_embed_streams")
+    return x
+
+
+def hyper_step(x: torch.Tensor, y: torch.Tensor | None,
+               mix: torch.Tensor | None, out_w: torch.Tensor | None,
+               in_w: torch.Tensor | None, norm_w: torch.Tensor | None,
+               eps: float) -> torch.Tensor | None:
+    """One step of the stream mixer, in place on x [T, S, W] fp32.
+
+    With y [T, W] (a sublayer's output): every stream at once from the old
+    ones, x_r <- sum_s mix[s, r] x_s + out_w[r] y.  With in_w [S]: returns
+    u = sum_r in_w[r] x_r of the (updated) streams as fp32 [T, W], RMS-normed
+    as u / rms(u) * (1 + norm_w) when norm_w is given.  mix [S, S], out_w and
+    in_w are fp32."""
+    T, S, W = x.shape
+    if not _gpu(x):
+        if y is not None:
+            x.copy_(torch.einsum("sr,tsw->trw", mix.float(), x)
+                    + out_w.float()[None, :, None] * y.float()[:, None, :])
+        if in_w is None:
+            return None
+        u = torch.einsum("s,tsw->tw", in_w.float(), x)
+        if norm_w is not None:
+            u = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) \
+                * (1.0 + norm_w.float())
+        return u
+    n = torch.empty(T, W, dtype=torch.float32, device=x.device) \
+        if in_w is not None else None
+    ref = y if y is not None else norm_w
+    rc = _L().afm_hyper_step(
+        _lib.ptr(x), _lib.ptr(y), _rowstride(y) if y is not None else 0,
+        _lib.ptr(mix), _lib.ptr(out_w), _lib.ptr(in_w), _lib.ptr(norm_w),
+        float(eps), _lib.ptr(n), T, S, W, 1 if norm_w is not None else 0,
+        _code(ref) if ref is not None else 1, _lib.cur_stream())
+    _lib.check(rc, "afm_hyper_step")
+    return n
+
+
+def canon_conv(n: torch.Tensor, w: torch.Tensor, state: torch.Tensor, md,
+               out_dtype: torch.dtype) -> torch.Tensor:
+    """h[t] = n[t] + sum_j w[:, j] n[t - (taps-1-j)]: a depthwise causal
+    convolution over time added to its own input.  n [T, W] fp32 packed
+    chunks, w [W, taps].  Inputs from before a chunk come from the sequence's
+    slot of `state` [slots, max(taps-1, 1), W] fp32 (oldest first), inputs
+    before position 0 are zero; afterwards the slot holds the sequence's last
+    taps-1 inputs.  Returns h in out_dtype."""
+    T, W = n.shape
+    taps = w.shape[1]
+    B = md.q_start.numel()
+    if not _gpu(n):
+        out = torch.empty(T, W, dtype=torch.float32)
+        cu, qs, sl = (md.cu_seqlens.tolist(), md.q_start.tolist(),
+                      md.state_slots.tolist())
+        wf = w.float()
+        for b in range(B):
+            r0, r1 = cu[b], cu[b + 1]
+            if r1 == r0:
+                continue
+            hist = state[sl[b]][:taps - 1].clone()
+            if qs[b] < taps - 1:      # places before position 0
+                hist[:taps - 1 - qs[b]] = 0.0
+            cat = torch.cat([hist, n[r0:r1]], 0)
+            acc = n[r0:r1].clone()
+            for j in range(taps):
+                acc += wf[:, j] * cat[j:j + r1 - r0]
+            out[r0:r1] = acc
+            if taps > 1:
+                state[sl[b]][:taps - 1] = cat[-(taps - 1):]
+        return out.to(out_dtype)
+    h = torch.empty(T, W, dtype=out_dtype, device=n.device)
+    if w.dtype != out_dtype:
+        raise TypeError("canon_conv: weights must be in the output dtype")
+    rc = _L().afm_canon_conv(
+        _lib.ptr(h), _lib.ptr(n), _lib.ptr(w), _lib.ptr(state),
+        _lib.ptr(md.row_seq), _lib.ptr(md.cu_seqlens), _lib.ptr(md.q_start),
+        _lib.ptr(md.state_slots), T, B, W, taps, _code(h), _lib.cur_stream())
+    _lib.check(rc, "afm_canon_conv")
+    return h
+
+
+def rotate_pairs(x: torch.Tensor, positions: torch.Tensor,
+                 inv_freq: torch.Tensor) -> torch.Tensor:
+    """Interleaved rotary embedding of the leading 2*len(inv_freq) elements
+    of the last axis (element 2i pairs with 2i+1; angle = position * f_i);
+    x [T, ..., d] fp32, CPU helper of latent_prep."""
+    r = 2 * inv_freq.numel()
+    ang = positions.float()[:, None] * inv_freq.float()[None]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [r // 2]
+    c, s = ang.cos().view(shape), ang.sin().view(shape)
+    u, v = x[..., 0:r:2], x[..., 1:r:2]
+    out = x.clone()
+    out[..., 0:r:2] = u * c - v * s
+    out[..., 1:r:2] = v * c + u * s
+    return out
+
+
+def latent_prep(q: torch.Tensor, dkv: torch.Tensor, qa: torch.Tensor,
+                norm_w: torch.Tensor, eps: float,
+                inv_freq: torch.Tensor | None, positions: torch.Tensor,
+                kcache: torch.Tensor, slots: torch.Tensor, heads: int,
+                dim: int) -> torch.Tensor:
+    """Row steps of latent attention.  dkv [T, R + rd] (may be a strided
+    view) holds the latent and one rotary key part: the latent is RMS-normed
+    with a plain weight, the key part rotated (interleaved pairs on its first
+    2*len(inv_freq) elements), and [latent | key part] is appended to the key
+    pages kcache [P, 1, page, R + rd] at `slots`.  q [T, H*(dim + rd)] holds
+    per head [unrotated | rotary part]; qa [H, T, R] is the unrotated part
+    already carried into latent space.  Returns the attention queries
+    [T, H*(R + rd)] = per head [qa | rotated rotary part]."""
+    T = q.shape[0]
+    H = heads
+    R = norm_w.numel()
+    rd = dkv.shape[1] - R
+    dkc = R + rd
+    page = kcache.shape[2]
+    rot = 2 * inv_freq.numel() if inv_freq is not None else 0
+    if not _gpu(q):
+        d = dkv.float()
+        c = d[:, :R] * torch.rsqrt(d[:, :R].pow(2).mean(-1, keepdim=True)
+                                   + eps) * norm_w.float()
+        kr = d[:, R:]
+        qr = q.float().view(T, H, dim + rd)[..., dim:]
+        if rot:
+            kr = rotate_pairs(kr, positions, inv_freq)
+            qr = rotate_pairs(qr, positions, inv_freq)
+        pg = torch.div(slots, page, rounding_mode="floor")
+        off = slots - pg * page
+        kcache[pg, 0, off] = torch.cat([c, kr], 1).to(kcache.dtype)
+        qf = torch.cat([qa.float().transpose(0, 1), qr], -1)
+        return qf.reshape(T, H * dkc).to(q.dtype)
+    qf = torch.empty(T, H * dkc, dtype=q.dtype, device=q.device)
+    qa = qa.contiguous()
+    rc = _L().afm_latent_prep(
+        _lib.ptr(qf), _lib.ptr(kcache), _lib.ptr(q), _rowstride(q),
+        _lib.ptr(dkv), _rowstride(dkv), _lib.ptr(qa), _lib.ptr(norm_w),
+        _lib.ptr(inv_freq), _lib.ptr(positions), _lib.ptr(slots), float(eps),
+        T, H, dim, rd, R, rot, _code(q), _lib.cur_stream())
+    _lib.check(rc, "afm_latent_prep")
+    return qf
+
+
+def gate_heads(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """out[t, h*dv + d] = o[h, t, d] * sigmoid(gate[t, h*dv + d]): per-head
+    results [H, T, dv] back to token rows, times an element-wise output gate
+    (logits [T, H*dv], may be a strided view)."""
+    H, T, dv = o.shape
+    if not _gpu(o):
+        return (o.float().transpose(0, 1).reshape(T, H * dv)
+                * torch.sigmoid(gate.float())).to(o.dtype)
+    o = o.contiguous()
+    out = torch.empty(T, H * dv, dtype=o.dtype, device=o.device)
+    rc = _L().afm_gate_heads(_lib.ptr(out), _lib.ptr(o), _lib.ptr(gate),
+                             _rowstride(gate), T, H, dv, _code(o),
+                             _lib.cur_stream())
+    _lib.check(rc, "afm_gate_heads")
+    return out
+
+
+def relu2(z: torch.Tensor) -> torch.Tensor:
+    """max(z, 0)^2, element-wise; z [T, F] may be a strided view."""
+    T, F = z.shape
+    if not _gpu(z):
+        return torch.relu(z.float()).pow(2).to(z.dtype)
+    out = torch.empty(T, F, dtype=z.dtype, device=z.device)
+    rc = _L().afm_relu2(_lib.ptr(out), _lib.ptr(z), _rowstride(z), T, F,
+                        _code(z), _lib.cur_stream())
+    _lib.check(rc, "afm_relu2")
     return out
