@@ -228,6 +228,191 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
   }
 }
 
+// ------------------------------------------------ single rows, many heads
+// One token's query heads of a K/V group as the rows of the MFMA tiles: the
+// case of decode steps when many heads share one K/V head (16 heads on one
+// latent row are exactly one 16-row tile), where a lane-per-key walk spends
+// its time on H dot products per key.  Workgroup = (token, K/V group x block
+// of 64 heads, key split); wave w owns heads 16w..16w+15 of the block and all
+// four waves stage the 64-key tiles.  Key splits cover multiples of 64 keys;
+// with nsplit > 1 unnormalised outputs and (max, sum) go to part_o [T, H,
+// nsplit, dv] / part_ml [T, H, nsplit, 2] for the split merge.
+template <int DKC, int DVT, bool VEC>
+__global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
+    u16* __restrict__ out, const u16* __restrict__ q,
+    const u16* __restrict__ kc, const u16* __restrict__ vc,
+    const i32* __restrict__ bt, const i32* __restrict__ row_seq,
+    const i32* __restrict__ positions, float scale, int H, int G, int dk,
+    int dv, int page, int maxp, int chunk, int window, i64 ldq, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml, AttnExtra ex) {
+  constexpr int KS = DKC * 32 + 8;
+  constexpr int VS = 72;
+  __shared__ u16 k_lds[64 * KS];
+  __shared__ u16 v_lds[DVT * 16 * VS];
+  __shared__ u16 p_lds[4 * 16 * VS];
+
+  const int t = blockIdx.x, sp = blockIdx.z;
+  const int hpg = H / G, nhb = (hpg + 63) / 64;
+  const int g = blockIdx.y / nhb, hb = blockIdx.y % nhb;
+  const int hbase = g * hpg + hb * 64;
+  const int nrows = min(64, hpg - hb * 64);
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  const i32* btr = bt + (size_t)row_seq[t] * maxp;
+  int lo = 0, hi = pos;
+  if (chunk > 0) lo = (pos / chunk) * chunk;
+  if (window > 0) lo = max(lo, pos - window + 1);
+  if (nsplit > 1) {   // this workgroup's share of [lo, pos]; may be empty
+    const int per = ((pos - lo + nsplit) / nsplit + 63) & ~63;
+    lo += sp * per;
+    hi = min(pos, lo + per - 1);
+  }
+  const int wrow0 = wid * 16;
+  const bool wave_live = wrow0 < nrows;
+
+  s16x8 q_frag[DKC];
+  {
+    const int head = hbase + min(wrow0 + (lane & 15), nrows - 1);
+    const u16* qr = q + (size_t)t * ldq + (size_t)head * dk;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c)
+      q_frag[c] = load8<VEC>(qr, c * 32 + (lane >> 4) * 8, dk);
+  }
+  float m[4], l[4], r1v[4], r2v[4];
+  f32x4 o_acc[DVT];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int hr = wrow0 + (lane >> 4) * 4 + r;
+    const int head = hbase + min(hr, nrows - 1);
+    const bool sk = ex.sink && sp == 0 && hr < nrows;   // first split only
+    m[r] = sk ? ex.sink[head] : AF_NEG_INF;
+    l[r] = sk ? 1.f : 0.f;
+    r1v[r] = ex.r1 ? ex.r1[head] : 0.f;
+    r2v[r] = ex.r1 ? ex.r2[head] : 0.f;
+  }
+#pragma unroll
+  for (int dt = 0; dt < DVT; ++dt) o_acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  u16* pw = p_lds + wid * 16 * VS;
+  const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
+
+  for (int kv0 = lo; kv0 <= hi; kv0 += 64) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * DKC * 4; i += 256) {
+      const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
+      const int j = kv0 + tok;
+      s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (j <= hi) {
+        const u16* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
+        v8 = load8<VEC>(kr, e0, dk);
+      }
+      *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
+    }
+    for (int i = threadIdx.x; i < 32 * DVT * 2; i += 256) {
+      const int tp = i % 32, e0 = (i / 32) * 8;
+      const int j0 = kv0 + tp * 2;
+      s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
+      if (j0 <= hi)
+        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * ex.ldv, e0, dv);
+      if (j0 + 1 <= hi)
+        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * ex.ldv, e0, dv);
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
+                                ((uint32_t)(unsigned short)c8[jj] << 16);
+        *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
+      }
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+
+    f32x4 s_acc[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      s_acc[st] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const u16* krow = k_lds + (st * 16 + (lane & 15)) * KS + (lane >> 4) * 8;
+#pragma unroll
+      for (int c = 0; c < DKC; ++c) {
+        const s16x8 kf = *reinterpret_cast<const s16x8*>(krow + c * 32);
+        s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            as_bf16x8(q_frag[c]), as_bf16x8(kf), s_acc[st], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sr[4];
+      float tmax = AF_NEG_INF;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int j = kv0 + st * 16 + (lane & 15);
+        float sv = s_acc[st][r] * scale;
+        if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
+        if (ex.r1) sv -= attn_dist_bias(r1v[r], r2v[r], max(pos - j, 0));
+        sr[st] = (j <= hi) ? sv : AF_NEG_INF;
+        tmax = fmaxf(tmax, sr[st]);
+      }
+      tmax = group16_max_f32(tmax);
+      const float mn = fmaxf(m[r], tmax);
+      const float corr = (m[r] <= AF_NEG_INF) ? 0.f : __expf(m[r] - mn);
+      float psum = 0.f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        sr[st] = (sr[st] <= AF_NEG_INF) ? 0.f : __expf(sr[st] - mn);
+        psum += sr[st];
+        s_acc[st][r] = sr[st];
+      }
+      l[r] = l[r] * corr + group16_sum_f32(psum);
+      m[r] = mn;
+#pragma unroll
+      for (int dt = 0; dt < DVT; ++dt) o_acc[dt][r] *= corr;
+    }
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        pw[((lane >> 4) * 4 + r) * VS + st * 16 + (lane & 15)] = f2bf(s_acc[st][r]);
+    __builtin_amdgcn_wave_barrier();
+    const s16x8 pf0 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + (lane >> 4) * 8);
+    const s16x8 pf1 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + 32 + (lane >> 4) * 8);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) {
+      const u16* vrow = v_lds + (dt * 16 + (lane & 15)) * VS + (lane >> 4) * 8;
+      const s16x8 vf0 = *reinterpret_cast<const s16x8*>(vrow);
+      const s16x8 vf1 = *reinterpret_cast<const s16x8*>(vrow + 32);
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf0), as_bf16x8(vf0), o_acc[dt], 0, 0, 0);
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf1), as_bf16x8(vf1), o_acc[dt], 0, 0, 0);
+    }
+  }
+
+  if (!wave_live) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int hr = wrow0 + (lane >> 4) * 4 + r;
+    if (hr >= nrows) continue;
+    const size_t th = (size_t)t * H + hbase + hr;
+    if (nsplit == 1) {
+      const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DVT; ++dt) {
+        const int d = dt * 16 + (lane & 15);
+        if (d < dv) out[th * dv + d] = f2bf(o_acc[dt][r] * inv);
+      }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DVT; ++dt) {
+        const int d = dt * 16 + (lane & 15);
+        if (d < dv) part_o[(th * nsplit + sp) * dv + d] = o_acc[dt][r];
+      }
+      if ((lane & 15) == 0) {
+        part_ml[(th * nsplit + sp) * 2] = m[r];
+        part_ml[(th * nsplit + sp) * 2 + 1] = l[r];
+      }
+    }
+  }
+}
+
 }  // namespace
 
 // q [T, H*dk] bf16 rows at stride ldq; caches [P, G, page, dk|dv] bf16;
@@ -267,5 +452,45 @@ AF_EXPORT int afm_attn_prefill_mfma(
   else if (vec) APM(4, 8, true);
   else APM(4, 8, false);
 #undef APM
+  return af_last_err();
+}
+
+// One row per token (decode steps): q [T, H*dk] at stride ldq, position and
+// sequence of every row in positions / row_seq.  The caller merges the key
+// splits (afm_attn_split_combine) when nsplit > 1.
+AF_EXPORT int afm_attn_heads_mfma(
+    void* out, const void* q, const void* kc, const void* vc, const void* bt,
+    const void* row_seq, const void* positions, float scale, int T, int H,
+    int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
+    int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
+    const void* r1, const void* r2, i64 ldv, void* stream) {
+  if (T == 0) return 0;
+  if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
+  if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
+  if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
+  const bool vec = (dk % 8 == 0) && (dv % 8 == 0) && (ldq % 8 == 0) &&
+                   (ldv % 8 == 0) &&
+                   ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&
+                   ((uintptr_t)vc % 16 == 0);
+  if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
+  const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
+                     cap, ldv};
+  const int hpg = H / G;
+  dim3 grid(T, G * ((hpg + 63) / 64), nsplit), blk(256);
+  hipStream_t s = (hipStream_t)stream;
+#define AHM(DKC, DVT, VEC)                                                     \
+  attn_heads_mfma_kernel<DKC, DVT, VEC><<<grid, blk, 0, s>>>(                  \
+      (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,                \
+      (const i32*)bt, (const i32*)row_seq, (const i32*)positions, scale, H, G, \
+      dk, dv, page, maxp, chunk, window, ldq, nsplit, (float*)part_o,          \
+      (float*)part_ml, ex)
+  const bool small = dk <= 64 && dv <= 64;
+  if (dk > 320 || dv > 256) AHM(18, 32, true);
+  else if (dk > 128 || dv > 128) AHM(10, 16, true);
+  else if (small && vec) AHM(2, 4, true);
+  else if (small) AHM(2, 4, false);
+  else if (vec) AHM(4, 8, true);
+  else AHM(4, 8, false);
+#undef AHM
   return af_last_err();
 }

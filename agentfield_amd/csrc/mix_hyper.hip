@@ -83,12 +83,27 @@ __global__ void __launch_bounds__(256) embed_streams_kernel(
 // With in: the next sublayer's input is read out, u = sum_r in[r] x_r, and
 // left in `n` either as it is (norm_mode 0) or as u / rms(u) * (1 + w)
 // (norm_mode 1).  MS bounds the stream count; V columns per access.
+//
+// With a convolution tail (steps of one row per sequence, row t = sequence
+// t): the normed row goes straight through the input convolution, h = n +
+// sum_j w[:, j] n_(t - (taps-1-j)) with the earlier inputs taken from the
+// sequence's slot, h leaves in the storage dtype, and the slot moves on by
+// one input; `n` is then scratch.
+struct ConvTail {
+  const void* w;       // [W, taps] storage dtype, null: no tail
+  float* state;        // [slots, max(taps-1, 1), W]
+  const i32* sslot;    // [T]
+  const i32* pos;      // [T] position of the row
+  void* h;             // [T, W] storage dtype
+  int taps;
+};
+
 template <typename S, int MS, int V>
 __global__ void __launch_bounds__(256) hyper_step_kernel(
     float* __restrict__ x, const S* __restrict__ y, i64 ldy,
     const float* __restrict__ mixm, const float* __restrict__ outv,
     const float* __restrict__ inv, const S* __restrict__ normw, float eps,
-    float* __restrict__ n, int ns, int W, int norm_mode) {
+    float* __restrict__ n, int ns, int W, int norm_mode, ConvTail ct) {
   __shared__ float s_mix[MS * MS], s_in[MS], s_out[MS], red[4];
   const int t = blockIdx.x;
   if (threadIdx.x < MS * MS) {
@@ -153,7 +168,28 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
     ldv<S, V>(normw + c, w4);
 #pragma unroll
     for (int j = 0; j < V; ++j) u[j] *= rinv * (1.0f + w4[j]);
-    stv<float, V>(nr + c, u);
+    if (!ct.w) {
+      stv<float, V>(nr + c, u);
+      continue;
+    }
+    const int hist = ct.taps - 1;
+    const int p = ct.pos[t];
+    float* st = ct.state + (size_t)ct.sslot[t] * (hist > 0 ? hist : 1) * W;
+    const S* cw = (const S*)ct.w + (size_t)c * ct.taps;
+    float acc[4];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = u[j] + ldf<S>(cw + j * ct.taps + hist) * u[j];
+    // place i of the slot holds the input of position p - hist + i; walking
+    // from the oldest, each is weighed by tap i and moved one place down
+    for (int i = 0; i < hist; ++i) {
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p - hist + i >= 0) ldv<float, V>(st + (size_t)i * W + c, v);
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[j] += ldf<S>(cw + j * ct.taps + i) * v[j];
+      if (i > 0) stv<float, V>(st + (size_t)(i - 1) * W + c, v);
+    }
+    if (hist > 0) stv<float, V>(st + (size_t)(hist - 1) * W + c, u);
+    stv<S, V>((S*)ct.h + (size_t)t * W + c, acc);
   }
 }
 
@@ -162,32 +198,34 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
 // convolution added to its own input.  Rows before the chunk come from the
 // sequence's slot of `state` [slots, taps-1, W] fp32 (oldest first), rows
 // before position 0 are zero.  One workgroup per (row, 256 channels).
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) canon_conv_kernel(
     S* __restrict__ h, const float* __restrict__ n, const S* __restrict__ w,
     const float* __restrict__ state, const i32* __restrict__ row_seq,
     const i32* __restrict__ cu, const i32* __restrict__ q_start,
     const i32* __restrict__ sslot, int W, int taps) {
   const int t = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * V;
   if (c >= W) return;
   const int b = row_seq[t];
   const int r = t - cu[b];
   const int p = q_start[b] + r;
   const int hist = taps - 1;
   const float* st = state + (size_t)sslot[b] * (hist > 0 ? hist : 1) * W;
-  const float cur = n[(size_t)t * W + c];
-  float acc = cur;
-  for (int j = 0; j < taps; ++j) {
-    const int k = hist - j;                  // rows back
-    float v = 0.f;
-    if (k == 0) v = cur;
-    else if (p - k < 0) v = 0.f;
-    else if (r - k >= 0) v = n[(size_t)(t - k) * W + c];
-    else v = st[(size_t)(hist + r - k) * W + c];
-    acc += ldf<S>(w + (size_t)c * taps + j) * v;
+  const S* cw = w + (size_t)c * taps;
+  float cur[4], acc[4];
+  ldv<float, V>(n + (size_t)t * W + c, cur);
+#pragma unroll
+  for (int j = 0; j < V; ++j) acc[j] = cur[j] + ldf<S>(cw + j * taps + hist) * cur[j];
+  for (int k = 1; k <= hist; ++k) {          // k rows back, tap hist - k
+    if (p - k < 0) break;                    // before the sequence: zeros
+    float v[4];
+    if (r - k >= 0) ldv<float, V>(n + (size_t)(t - k) * W + c, v);
+    else ldv<float, V>(st + (size_t)(hist + r - k) * W + c, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] += ldf<S>(cw + j * taps + hist - k) * v[j];
   }
-  stf<S>(h + (size_t)t * W + c, acc);
+  stv<S, V>(h + (size_t)t * W + c, acc);
 }
 
 // After the convolution: the slot keeps the sequence's last taps-1 inputs.
@@ -286,19 +324,23 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(
 
 // out[t, h*dv + d] = o[h, t, d] * sigmoid(g[t, h*dv + d]): head-major
 // per-head results back to token rows, times the output gate.
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) gate_heads_kernel(
     S* __restrict__ out, const S* __restrict__ o, const S* __restrict__ g,
     i64 ldg, int T, int H, int dv) {
-  const i64 total = (i64)T * H * dv;
+  const int per = dv / V;
+  const i64 total = (i64)T * H * per;
   for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < total;
        i += (i64)gridDim.x * 256) {
-    const int d = (int)(i % dv);
-    const int h = (int)((i / dv) % H);
-    const i64 t = i / ((i64)dv * H);
-    const float gv = ldf<S>(g + t * ldg + (i64)h * dv + d);
-    const float ov = ldf<S>(o + ((i64)h * T + t) * dv + d);
-    stf<S>(out + i, ov / (1.0f + expf(-gv)));
+    const int d = (int)(i % per) * V;
+    const int h = (int)((i / per) % H);
+    const i64 t = i / ((i64)per * H);
+    float gv[4], ov[4];
+    ldv<S, V>(g + t * ldg + (i64)h * dv + d, gv);
+    ldv<S, V>(o + ((i64)h * T + t) * dv + d, ov);
+#pragma unroll
+    for (int j = 0; j < V; ++j) ov[j] = ov[j] / (1.0f + expf(-gv[j]));
+    stv<S, V>(out + (t * H + h) * dv + d, ov);
   }
 }
 
@@ -348,13 +390,13 @@ static int launch_hyper_step(float* x, const void* y, i64 ldy,
                              const float* mixm, const float* outv,
                              const float* inv, const void* normw, float eps,
                              float* n, int T, int ns, int W, int norm_mode,
-                             hipStream_t s) {
+                             ConvTail ct, hipStream_t s) {
   const bool vec = W % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(n) &&
-                   al16(y) && al16(normw);
+                   al16(y) && al16(normw) && al16(ct.state) && al16(ct.h);
 #define HS(MS, V)                                                            \
   hyper_step_kernel<S, MS, V><<<T, 256, 0, s>>>(                             \
       x, (const S*)y, ldy, mixm, outv, inv, (const S*)normw, eps, n, ns, W,  \
-      norm_mode)
+      norm_mode, ct)
   if (ns <= 4) { if (vec) HS(4, 4); else HS(4, 1); }
   else if (ns <= 8) { if (vec) HS(8, 4); else HS(8, 1); }
   else { if (vec) HS(16, 4); else HS(16, 1); }
@@ -364,24 +406,33 @@ static int launch_hyper_step(float* x, const void* y, i64 ldy,
 
 // x [T, ns, W] fp32 in place; y [T, W] at row stride ldy (or null); mixm
 // [ns, ns] indexed [from, to], outv / inv [ns] fp32; normw [W]; n [T, W] fp32.
+// conv_w [W, taps] switches the convolution tail on (one row per sequence;
+// needs the norm): conv_state [slots, max(taps-1, 1), W] fp32, sslot / pos
+// [T], h [T, W] in the storage dtype.
 AF_EXPORT int afm_hyper_step(void* x, const void* y, i64 ldy, const void* mixm,
                              const void* outv, const void* inv,
                              const void* normw, float eps, void* n, int T,
-                             int ns, int W, int norm_mode, int dt,
+                             int ns, int W, int norm_mode, const void* conv_w,
+                             void* conv_state, const void* sslot,
+                             const void* pos, int taps, void* h, int dt,
                              void* stream) {
   if (T == 0) return 0;
   if (ns < 1 || ns > 16) return 9003;
   if (y && (!mixm || !outv)) return 9003;
   if (inv && (!n || (norm_mode == 1 && !normw))) return 9003;
+  if (conv_w && (!inv || norm_mode != 1 || taps < 1 || !conv_state || !sslot ||
+                 !pos || !h)) return 9003;
+  const ConvTail ct{conv_w, (float*)conv_state, (const i32*)sslot,
+                    (const i32*)pos, h, taps};
   hipStream_t s = (hipStream_t)stream;
   if (dt == 0)
     return launch_hyper_step<u16>((float*)x, y, ldy, (const float*)mixm,
         (const float*)outv, (const float*)inv, normw, eps, (float*)n, T, ns, W,
-        norm_mode, s);
+        norm_mode, ct, s);
   if (dt == 1)
     return launch_hyper_step<float>((float*)x, y, ldy, (const float*)mixm,
         (const float*)outv, (const float*)inv, normw, eps, (float*)n, T, ns, W,
-        norm_mode, s);
+        norm_mode, ct, s);
   return 9002;
 }
 
@@ -394,19 +445,17 @@ AF_EXPORT int afm_canon_conv(void* h, const void* n, const void* w,
   if (T == 0) return 0;
   if (taps < 1) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(T, (W + 255) / 256);
-  if (dt == 0)
-    canon_conv_kernel<u16><<<grid, 256, 0, s>>>(
-        (u16*)h, (const float*)n, (const u16*)w, (const float*)state,
-        (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
-        (const i32*)sslot, W, taps);
-  else if (dt == 1)
-    canon_conv_kernel<float><<<grid, 256, 0, s>>>(
-        (float*)h, (const float*)n, (const float*)w, (const float*)state,
-        (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
-        (const i32*)sslot, W, taps);
-  else
-    return 9002;
+  const bool vec = W % 4 == 0 && al16(h) && al16(n) && al16(state);
+  dim3 grid(T, vec ? (W / 4 + 255) / 256 : (W + 255) / 256);
+#define CC(S, V)                                                              \
+  canon_conv_kernel<S, V><<<grid, 256, 0, s>>>(                               \
+      (S*)h, (const float*)n, (const S*)w, (const float*)state,               \
+      (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,               \
+      (const i32*)sslot, W, taps)
+  if (dt == 0) { if (vec) CC(u16, 4); else CC(u16, 1); }
+  else if (dt == 1) { if (vec) CC(float, 4); else CC(float, 1); }
+  else return 9002;
+#undef CC
   if (taps > 1)
     canon_state_kernel<<<dim3(B, (W + 255) / 256), 256, 0, s>>>(
         (float*)state, (const float*)n, (const i32*)cu, (const i32*)q_start,
@@ -443,16 +492,17 @@ AF_EXPORT int afm_gate_heads(void* out, const void* o, const void* g, i64 ldg,
                              int T, int H, int dv, int dt, void* stream) {
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const i64 total = (i64)T * H * dv;
-  const int grid = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
-  if (dt == 0)
-    gate_heads_kernel<u16><<<grid, 256, 0, s>>>((u16*)out, (const u16*)o,
-                                                (const u16*)g, ldg, T, H, dv);
-  else if (dt == 1)
-    gate_heads_kernel<float><<<grid, 256, 0, s>>>(
-        (float*)out, (const float*)o, (const float*)g, ldg, T, H, dv);
-  else
-    return 9002;
+  const bool vec = dv % 4 == 0 && ldg % 4 == 0 && al16(out) && al16(o) &&
+                   al16(g);
+  const i64 total = (i64)T * H * (vec ? dv / 4 : dv);
+  const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+#define GH(S, V)                                                              \
+  gate_heads_kernel<S, V><<<grid, 256, 0, s>>>((S*)out, (const S*)o,          \
+                                               (const S*)g, ldg, T, H, dv)
+  if (dt == 0) { if (vec) GH(u16, 4); else GH(u16, 1); }
+  else if (dt == 1) { if (vec) GH(float, 4); else GH(float, 1); }
+  else return 9002;
+#undef GH
   return af_last_err();
 }
 

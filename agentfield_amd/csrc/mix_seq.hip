@@ -739,6 +739,23 @@ AF_EXPORT int afm_masked_attention(
   return 9002;
 }
 
+// out [T*H, dv] bf16 from part_o [T*H, nsplit, dv] / part_ml [T*H, nsplit, 2].
+AF_EXPORT int afm_attn_split_combine(void* out, const void* part_o,
+                                     const void* part_ml, int n_rh, int nsplit,
+                                     int dv, int dt, void* stream) {
+  if (n_rh == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    attn_split_combine_kernel<u16><<<(n_rh + 3) / 4, 256, 0, s>>>(
+        (u16*)out, (const float*)part_o, (const float*)part_ml, n_rh, nsplit, dv);
+  else if (dt == 1)
+    attn_split_combine_kernel<float><<<(n_rh + 3) / 4, 256, 0, s>>>(
+        (float*)out, (const float*)part_o, (const float*)part_ml, n_rh, nsplit, dv);
+  else
+    return 9002;
+  return af_last_err();
+}
+
 template <typename S>
 static int launch_scan(float* out, float* state, const void* q, const void* k,
                        const void* v, const void* zl, const float* zbias,

@@ -386,16 +386,17 @@ class FugevikForCausalLM(nn.Module):
         back = (None, None, None)
         for run, L in enumerate(self.layers):
             port = L.port1
-            n = sm.hyper_step(x, *back, port.inw, port.norm, eps)
-            h = sm.canon_conv(n, port.canon, cache.state["canon1"][run], md,
-                              dt)
+            h = sm.hyper_conv_step(x, *back, port.inw, port.norm, eps,
+                                   port.canon, cache.state["canon1"][run], md,
+                                   positions, dt)
             y = L.mixer(h, cache, run, md, positions)
             back = (y, port.mix, port.outw)
             if L.mlp is not None:
                 port = L.port2
-                n = sm.hyper_step(x, *back, port.inw, port.norm, eps)
-                h = sm.canon_conv(n, port.canon,
-                                  cache.state["canon2"][run], md, dt)
+                h = sm.hyper_conv_step(x, *back, port.inw, port.norm, eps,
+                                       port.canon,
+                                       cache.state["canon2"][run], md,
+                                       positions, dt)
                 back = (L.mlp(h), port.mix, port.outw)
             if self.record_runs is not None:
                 self.record_runs.append(

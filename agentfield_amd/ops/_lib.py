@@ -152,6 +152,9 @@ def _mix_sigs() -> dict:
                                      i, p],
             "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i,
                                       i, i, i, i, i, i64, p, f, p, p, i64, p],
+            "afm_attn_heads_mfma": [p, p, p, p, p, p, p, f, i, i, i, i, i, i,
+                                    i, i, i, i64, i, p, p, p, f, p, p, i64, p],
+            "afm_attn_split_combine": [p, p, p, i, i, i, i, p],
             "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
                                 i, i, i, i, i, i64, i64, i64, i64, i, p],
         },
@@ -171,7 +174,8 @@ def _mix_sigs() -> dict:
         },
         "hyper": {
             "afm_embed_streams": [p, p, p, i, i, i, i, p],
-            "afm_hyper_step": [p, p, i64, p, p, p, p, f, p, i, i, i, i, i, p],
+            "afm_hyper_step": [p, p, i64, p, p, p, p, f, p, i, i, i, i, p, p,
+                               p, p, i, p, i, p],
             "afm_canon_conv": [p, p, p, p, p, p, p, p, i, i, i, i, i, p],
             "afm_latent_prep": [p, p, p, i64, p, i64, p, p, p, p, p, f, i, i,
                                 i, i, i, i, i, p],

@@ -31,6 +31,9 @@ _DT = {torch.bfloat16: 0, torch.float32: 1}
 # a step whose longest row chunk reaches this many rows runs bf16 attention
 # through the MFMA tile kernel; shorter steps (decode) use one wave per row
 MFMA_MIN_ROWS = 16
+# single rows (decode) with at least this many query heads per K/V head run
+# bf16 attention with the heads as matrix-core rows
+HEADS_MFMA_MIN = 8
 _SKINNY = os.environ.get("AF_MIX_SKINNY", "0") == "1"
 
 
@@ -284,10 +287,37 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
         if rc != 9004:          # 9004: no tile kernel for this head geometry
             _lib.check(rc, "afm_attn_prefill_mfma")
             return out
-    # few rows and many visible keys: cut the keys over several workgroups
-    # (about 2048 in flight) and merge the partial softmaxes
     reach = min(x for x in (chunk, window, md.block_table.shape[1] * page)
                 if x > 0)
+    if (q.dtype == torch.bfloat16 and H // G >= HEADS_MFMA_MIN and dk <= 576
+            and dv <= 512):
+        # single rows whose many heads share a K/V head: the heads are the
+        # rows of the matrix-core tiles; key splits of 64-key multiples
+        wgs = T * G * -(-(H // G) // 64)
+        nsplit = max(1, min(16, 2048 // max(1, wgs), -(-reach // 64)))
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = torch.empty(T, H, nsplit, dv, dtype=torch.float32,
+                                 device=q.device)
+            part_ml = torch.empty(T, H, nsplit, 2, dtype=torch.float32,
+                                  device=q.device)
+        rc = _L().afm_attn_heads_mfma(
+            _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vsrc),
+            _lib.ptr(md.block_table), _lib.ptr(md.row_seq),
+            _lib.ptr(positions), float(scale), T, H, G, dk, dv, page,
+            md.block_table.shape[1], int(chunk), int(window), _rowstride(q),
+            nsplit, _lib.ptr(part_o), _lib.ptr(part_ml), *extra,
+            _lib.cur_stream())
+        if rc != 9004:
+            _lib.check(rc, "afm_attn_heads_mfma")
+            if nsplit > 1:
+                rc = _L().afm_attn_split_combine(
+                    _lib.ptr(out), _lib.ptr(part_o), _lib.ptr(part_ml), T * H,
+                    nsplit, dv, _code(q), _lib.cur_stream())
+                _lib.check(rc, "afm_attn_split_combine")
+            return out
+    # few rows and many visible keys: cut the keys over several workgroups
+    # (about 2048 in flight) and merge the partial softmaxes
     per_wg_heads = min(8, max(1, H // G))
     wgs = T * G * -(-(H // G) // per_wg_heads)
     nsplit = max(1, min(8, 2048 // max(1, wgs), reach // 128))
@@ -929,7 +959,7 @@ def embed_streams(ids: torch.Tensor, table: torch.Tensor,
 def hyper_step(x: torch.Tensor, y: torch.Tensor | None,
                mix: torch.Tensor | None, out_w: torch.Tensor | None,
                in_w: torch.Tensor | None, norm_w: torch.Tensor | None,
-               eps: float) -> torch.Tensor | None:
+               eps: float, _tail: tuple | None = None) -> torch.Tensor | None:
     """One step of the stream mixer, in place on x [T, S, W] fp32.
 
     With y [T, W] (a sublayer's output): every stream at once from the old
@@ -952,13 +982,37 @@ def hyper_step(x: torch.Tensor, y: torch.Tensor | None,
     n = torch.empty(T, W, dtype=torch.float32, device=x.device) \
         if in_w is not None else None
     ref = y if y is not None else norm_w
+    h = None
+    tail = (None, None, None, None, 0, None)
+    if _tail is not None:
+        conv_w, state, md, positions = _tail
+        h = torch.empty(T, W, dtype=conv_w.dtype, device=x.device)
+        tail = (_lib.ptr(conv_w), _lib.ptr(state), _lib.ptr(md.state_slots),
+                _lib.ptr(positions), conv_w.shape[1], _lib.ptr(h))
     rc = _L().afm_hyper_step(
         _lib.ptr(x), _lib.ptr(y), _rowstride(y) if y is not None else 0,
         _lib.ptr(mix), _lib.ptr(out_w), _lib.ptr(in_w), _lib.ptr(norm_w),
         float(eps), _lib.ptr(n), T, S, W, 1 if norm_w is not None else 0,
-        _code(ref) if ref is not None else 1, _lib.cur_stream())
+        *tail, _code(ref) if ref is not None else 1, _lib.cur_stream())
     _lib.check(rc, "afm_hyper_step")
-    return n
+    return n if h is None else h
+
+
+def hyper_conv_step(x: torch.Tensor, y: torch.Tensor | None,
+                    mix: torch.Tensor | None, out_w: torch.Tensor | None,
+                    in_w: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                    conv_w: torch.Tensor, state: torch.Tensor, md,
+                    positions: torch.Tensor,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """hyper_step (write y in, read the next input out, norm) followed by
+    canon_conv: a sublayer's input in out_dtype.  Steps of one row per
+    sequence (decode) run as a single kernel on GPU."""
+    if _gpu(x) and not getattr(md, "is_prefill", True) \
+            and conv_w.dtype == out_dtype and norm_w.dtype == out_dtype:
+        return hyper_step(x, y, mix, out_w, in_w, norm_w, eps,
+                          _tail=(conv_w, state, md, positions))
+    n = hyper_step(x, y, mix, out_w, in_w, norm_w, eps)
+    return canon_conv(n, conv_w, state, md, out_dtype)
 
 
 def canon_conv(n: torch.Tensor, w: torch.Tensor, state: torch.Tensor, md,

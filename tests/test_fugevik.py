@@ -267,6 +267,44 @@ def test_input_conv_alone(device, dtype, taps):
         assert torch.equal(state[3].cpu(), seqs[0][T - taps + 1:])
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(3, 30, 3), (4, 64, 4), (1, 16, 1),
+                                   (7, 33, 5), (2, 8, 2)])
+def test_decode_step_fuses_input_conv(device, dtype, shape):
+    """Steps of one row per sequence (write, read, norm, convolution, slot
+    moved on in one kernel) against the separate ops, from position 0 on."""
+    S, W, taps = shape
+    B, steps = 3, 7
+    g = torch.Generator().manual_seed(S + W + taps)
+    d = lambda t: t.to(device)  # noqa: E731
+    mix = d(torch.eye(S) + 0.3 * torch.randn(S, S, generator=g))
+    outw, inw = d(torch.randn(S, generator=g)), d(torch.randn(S, generator=g))
+    nw = d((0.2 * torch.randn(W, generator=g)).to(dtype))
+    cw = d((0.5 * torch.randn(W, taps, generator=g)).to(dtype))
+    hist = max(taps - 1, 1)
+    st_a = torch.full((5, hist, W), 7.0, device=device)
+    st_b = st_a.clone()
+    starts = [0, 0, 0]
+    for step in range(steps):
+        x0 = torch.randn(B, S, W, generator=g)
+        y = d(torch.randn(B, W, generator=g).to(dtype))
+        md_a, pos = md_for([1] * B, [step] * B, [4, 1, 2], device)
+        md_b, _ = md_for([1] * B, [step] * B, [4, 1, 2], device, decode=True)
+        xa, xb = d(x0.clone()), d(x0.clone())
+        ha = sm.hyper_conv_step(xa, y, mix, outw, inw, nw, 1e-5, cw, st_a,
+                                md_a, pos, dtype)
+        hb = sm.hyper_conv_step(xb, y, mix, outw, inw, nw, 1e-5, cw, st_b,
+                                md_b, pos, dtype)
+        assert torch.equal(xa, xb)
+        assert (ha.float() - hb.float()).abs().max() < \
+            (1e-5 if dtype == torch.float32 else 5e-2)
+        if taps > 1:
+            keep = min(step + 1, taps - 1)      # places of real positions
+            assert (st_a[[4, 1, 2], hist - keep:] -
+                    st_b[[4, 1, 2], hist - keep:]).abs().max() < 1e-5
+
+
 def _attn_close(got, want, dtype):
     d = (got.to(F64).cpu() - want).pow(2).mean().sqrt()
     return float(d / want.pow(2).mean().sqrt()) < \
@@ -296,7 +334,10 @@ def _run_mixer(mod, layout, h, device, dtype, portions, page=8, decode_from=None
     (3, 10, 6, 14, 50, 33, 4),
     (2, 32, 16, 32, 144, 50, 16),     # wide rows: latent + key part = 160
     (2, 8, 8, 8, 328, 70, 8),         # wider than 320
-    (5, 6, 2, 6, 10, 7, 0)])          # nothing rotates
+    (5, 6, 2, 6, 10, 7, 0),           # nothing rotates
+    (9, 8, 8, 8, 24, 19, 8),          # many heads on the one latent row
+    (20, 16, 8, 12, 40, 0, 8),
+    (70, 4, 4, 4, 12, 30, 4)])        # more heads than one 64-row block
 def test_latent_attention_alone(device, dtype, shape):
     H, dim, rd, vd, R, window, dims = shape
     W, T = 28, 90
@@ -332,6 +373,7 @@ def test_latent_attention_alone(device, dtype, shape):
     (1, 1, 8, 8, 0, 0.0),
     (5, 5, 6, 10, 9, 30.0),
     (8, 1, 64, 64, 40, 1.5),
+    (24, 2, 8, 8, 21, 3.0),            # twelve heads per K/V head
     (4, 2, 40, 136, 64, 2.0)])         # values wider than 128
 def test_biased_attention_alone(device, dtype, shape):
     H, G, dim, vd, window, cap = shape
@@ -383,12 +425,13 @@ def test_feed_forward_alone(device, dtype):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("decode", [False, True])
-def test_window_edge_and_far_key(device, dtype, decode):
+@pytest.mark.parametrize("H", [2, 16])
+def test_window_edge_and_far_key(device, dtype, decode, H):
     """One loud key among hundreds: it is heard exactly while it is inside
     the window (distances window-1 and window apart), at a page's last and
     first place and far from the query; prompt rows and single rows."""
     page, T, window = 16, 400, 129
-    H, G, dk, dv = 2, 1, 8, 8
+    G, dk, dv = 1, 8, 8
     for loud in (0, 15, 16, 255, 270):
         pages = T // page
         kc = torch.zeros(pages + 2, G, page, dk, dtype=dtype, device=device)
@@ -401,8 +444,7 @@ def test_window_edge_and_far_key(device, dtype, decode):
                 loud + window, loud + window + 1]
         rows = [r for r in rows if r < T]
         q = torch.zeros(len(rows), H * dk, dtype=dtype, device=device)
-        q[:, 0] = 1.0
-        q[:, dk] = 1.0
+        q[:, 0::dk] = 1.0
         if decode:
             md = SimpleNamespace(
                 block_table=bt[None].repeat(len(rows), 1).to(device),
@@ -432,14 +474,16 @@ def test_window_edge_and_far_key(device, dtype, decode):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_sink_takes_weight_without_value(device, dtype):
+@pytest.mark.parametrize("H", [3, 9])
+def test_sink_takes_weight_without_value(device, dtype, H):
     """Equal scores everywhere: n keys share 1 - e^sink / (n + e^sink) of the
     weight; a huge sink silences the head, a tiny one changes nothing; the
     sink is not multiplied by the score scale."""
-    page, T, H, dk, dv = 8, 70, 3, 8, 6
+    page, T, dk, dv = 8, 70, 8, 6
     kc = torch.zeros(12, 1, page, dk, dtype=dtype, device=device)
     vc = torch.ones(12, 1, page, dv, dtype=dtype, device=device)
-    sink = torch.tensor([math.log(5.0), 40.0, -40.0], device=device)
+    sink = torch.tensor([math.log(5.0), 40.0, -40.0] + [0.0] * (H - 3),
+                        device=device)
     q = torch.zeros(T, H * dk, dtype=dtype, device=device)
     for decode in (False, True):
         md, pos = md_for([T], [0], [1], device, page=page, decode=decode)
