@@ -46,6 +46,53 @@ __device__ __forceinline__ s16x8 load8(const u16* row, int e0, int n) {
   return v;
 }
 
+// Stage one 64-key tile: K rows row-major into k_lds, V rows transposed into
+// v_lds ([d][token], token pairs packed into 32-bit writes).  The page walk
+// is done once per key (row_lds[tok] = row index in the pages, -1 for keys
+// past `last`), so the tile's loads depend on nothing but LDS and are issued
+// back to back.
+template <int DKC, int DVT, bool VEC>
+__device__ __forceinline__ void stage_kv_tile(
+    u16* k_lds, u16* v_lds, i32* row_lds, const u16* __restrict__ kc,
+    const u16* __restrict__ vc, const i32* __restrict__ btr, int kv0, int last,
+    int G, int g, int page, int dk, int dv, i64 ldv) {
+  constexpr int KS = DKC * 32 + 8;
+  constexpr int VS = 72;
+  if (threadIdx.x < 64) {
+    const int j = kv0 + threadIdx.x;
+    row_lds[threadIdx.x] =
+        j <= last ? (btr[j / page] * G + g) * page + (j % page) : -1;
+  }
+  __syncthreads();
+  constexpr int KIT = (64 * DKC * 4) / 256;
+#pragma unroll
+  for (int it = 0; it < KIT; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
+    const int row = row_lds[tok];
+    s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (row >= 0) v8 = load8<VEC>(kc + (size_t)row * dk, e0, dk);
+    *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
+  }
+  constexpr int VIT = (32 * DVT * 2 + 255) / 256;
+#pragma unroll
+  for (int it = 0; it < VIT; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i >= 32 * DVT * 2) break;
+    const int tp = i % 32, e0 = (i / 32) * 8;
+    const int ra = row_lds[tp * 2], rb = row_lds[tp * 2 + 1];
+    s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
+    if (ra >= 0) a = load8<VEC>(vc + (size_t)ra * ldv, e0, dv);
+    if (rb >= 0) c8 = load8<VEC>(vc + (size_t)rb * ldv, e0, dv);
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
+                              ((uint32_t)(unsigned short)c8[jj] << 16);
+      *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
+    }
+  }
+}
+
 template <int DKC, int DVT, bool VEC>
 __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
     u16* __restrict__ out, const u16* __restrict__ q,
@@ -60,6 +107,7 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
   __shared__ u16 v_lds[DVT * 16 * VS];
   __shared__ u16 p_lds[4 * 16 * VS];
   __shared__ float bias_lds[128];    // distance bias of this tile's distances
+  __shared__ i32 row_lds[64];        // page row of every key of the tile
 
   const int tile = blockIdx.x, h = blockIdx.y;
   const int g = h / (H / G);
@@ -106,33 +154,8 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
 
   for (int kv0 = lo; kv0 <= p_last; kv0 += 64) {
     __syncthreads();   // fragment reads of the previous tile are done
-    // ---- stage K: 64 tokens x DKC*4 groups of 8 ----
-    for (int i = threadIdx.x; i < 64 * DKC * 4; i += 256) {
-      const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
-      const int j = kv0 + tok;
-      s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (j <= p_last) {
-        const u16* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
-        v8 = load8<VEC>(kr, e0, dk);
-      }
-      *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
-    }
-    // ---- stage V transposed: token pairs -> one 32-bit write per d ----
-    for (int i = threadIdx.x; i < 32 * DVT * 2; i += 256) {
-      const int tp = i % 32, e0 = (i / 32) * 8;
-      const int j0 = kv0 + tp * 2;
-      s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
-      if (j0 <= p_last)
-        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * ex.ldv, e0, dv);
-      if (j0 + 1 <= p_last)
-        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * ex.ldv, e0, dv);
-#pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
-                                ((uint32_t)(unsigned short)c8[jj] << 16);
-        *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
-      }
-    }
+    stage_kv_tile<DKC, DVT, VEC>(k_lds, v_lds, row_lds, kc, vc, btr, kv0,
+                                 p_last, G, g, page, dk, dv, ex.ldv);
     // distance bias for every distance between a row and a key of the tile:
     // entry i is distance i + (p0 - kv0 - 63); keys ahead of a row are masked
     if (ex.r1 && threadIdx.x < 127) {
@@ -250,6 +273,7 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
   __shared__ u16 k_lds[64 * KS];
   __shared__ u16 v_lds[DVT * 16 * VS];
   __shared__ u16 p_lds[4 * 16 * VS];
+  __shared__ i32 row_lds[64];
 
   const int t = blockIdx.x, sp = blockIdx.z;
   const int hpg = H / G, nhb = (hpg + 63) / 64;
@@ -269,6 +293,16 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
   }
   const int wrow0 = wid * 16;
   const bool wave_live = wrow0 < nrows;
+  if (lo > hi && !(ex.sink && sp == 0)) {
+    // an empty split (the grid is sized for the longest reach): mark it and
+    // leave before touching queries or pages
+    for (int i = threadIdx.x; i < nrows; i += 256) {
+      const size_t th = (size_t)t * H + hbase + i;
+      part_ml[(th * nsplit + sp) * 2] = AF_NEG_INF;
+      part_ml[(th * nsplit + sp) * 2 + 1] = 0.f;
+    }
+    return;
+  }
 
   s16x8 q_frag[DKC];
   {
@@ -297,31 +331,8 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
 
   for (int kv0 = lo; kv0 <= hi; kv0 += 64) {
     __syncthreads();
-    for (int i = threadIdx.x; i < 64 * DKC * 4; i += 256) {
-      const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
-      const int j = kv0 + tok;
-      s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (j <= hi) {
-        const u16* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
-        v8 = load8<VEC>(kr, e0, dk);
-      }
-      *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
-    }
-    for (int i = threadIdx.x; i < 32 * DVT * 2; i += 256) {
-      const int tp = i % 32, e0 = (i / 32) * 8;
-      const int j0 = kv0 + tp * 2;
-      s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
-      if (j0 <= hi)
-        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * ex.ldv, e0, dv);
-      if (j0 + 1 <= hi)
-        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * ex.ldv, e0, dv);
-#pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
-                                ((uint32_t)(unsigned short)c8[jj] << 16);
-        *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
-      }
-    }
+    stage_kv_tile<DKC, DVT, VEC>(k_lds, v_lds, row_lds, kc, vc, btr, kv0, hi,
+                                 G, g, page, dk, dv, ex.ldv);
     __syncthreads();
     if (!wave_live) continue;
 

@@ -118,7 +118,12 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
   float* xr = x + (size_t)t * ns * W;
   float* nr = n ? n + (size_t)t * W : nullptr;
   float ss = 0.f;
-  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+  // the first KEEP column groups of a thread stay in registers across the
+  // row reduction; wider rows go through `n`
+  constexpr int KEEP = 4;
+  float held[KEEP][4];
+  int it = 0;
+  for (int c = threadIdx.x * V; c < W; c += 256 * V, ++it) {
     float xs[MS][4];
 #pragma unroll
     for (int s = 0; s < MS; ++s)
@@ -156,15 +161,29 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
         }
 #pragma unroll
       for (int j = 0; j < V; ++j) ss += u[j] * u[j];
-      stv<float, V>(nr + c, u);
+      if (norm_mode == 0 || it >= KEEP) stv<float, V>(nr + c, u);
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k)
+        if (k == it) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) held[k][j] = u[j];
+        }
     }
   }
   if (!inv || norm_mode == 0) return;
   const float rinv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)W + eps);
-  // every thread rescales the columns it wrote itself
-  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+  const int tail_pos = ct.w ? ct.pos[t] : 0;
+  const int tail_slot = ct.w ? ct.sslot[t] : 0;
+  it = 0;
+  for (int c = threadIdx.x * V; c < W; c += 256 * V, ++it) {
     float u[4], w4[4];
-    ldv<float, V>(nr + c, u);
+    if (it >= KEEP) ldv<float, V>(nr + c, u);   // columns this thread wrote
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k)
+      if (k == it) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) u[j] = held[k][j];
+      }
     ldv<S, V>(normw + c, w4);
 #pragma unroll
     for (int j = 0; j < V; ++j) u[j] *= rinv * (1.0f + w4[j]);
@@ -173,8 +192,8 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
       continue;
     }
     const int hist = ct.taps - 1;
-    const int p = ct.pos[t];
-    float* st = ct.state + (size_t)ct.sslot[t] * (hist > 0 ? hist : 1) * W;
+    const int p = tail_pos;
+    float* st = ct.state + (size_t)tail_slot * (hist > 0 ? hist : 1) * W;
     const S* cw = (const S*)ct.w + (size_t)c * ct.taps;
     float acc[4];
 #pragma unroll
@@ -198,34 +217,55 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
 // convolution added to its own input.  Rows before the chunk come from the
 // sequence's slot of `state` [slots, taps-1, W] fp32 (oldest first), rows
 // before position 0 are zero.  One workgroup per (row, 256 channels).
+constexpr int CONV_ROWS = 8;   // consecutive rows per workgroup: a row's
+                               // predecessors were just read by the same CU
+constexpr int CONV_REGT = 8;   // taps whose weights stay in registers
+
 template <typename S, int V>
 __global__ void __launch_bounds__(256) canon_conv_kernel(
     S* __restrict__ h, const float* __restrict__ n, const S* __restrict__ w,
     const float* __restrict__ state, const i32* __restrict__ row_seq,
     const i32* __restrict__ cu, const i32* __restrict__ q_start,
-    const i32* __restrict__ sslot, int W, int taps) {
-  const int t = blockIdx.x;
+    const i32* __restrict__ sslot, int T, int W, int taps) {
   const int c = (blockIdx.y * 256 + threadIdx.x) * V;
   if (c >= W) return;
-  const int b = row_seq[t];
-  const int r = t - cu[b];
-  const int p = q_start[b] + r;
   const int hist = taps - 1;
-  const float* st = state + (size_t)sslot[b] * (hist > 0 ? hist : 1) * W;
   const S* cw = w + (size_t)c * taps;
-  float cur[4], acc[4];
-  ldv<float, V>(n + (size_t)t * W + c, cur);
+  float wb[CONV_REGT][4];        // wb[k]: weight of the input k rows back
 #pragma unroll
-  for (int j = 0; j < V; ++j) acc[j] = cur[j] + ldf<S>(cw + j * taps + hist) * cur[j];
-  for (int k = 1; k <= hist; ++k) {          // k rows back, tap hist - k
-    if (p - k < 0) break;                    // before the sequence: zeros
-    float v[4];
-    if (r - k >= 0) ldv<float, V>(n + (size_t)(t - k) * W + c, v);
-    else ldv<float, V>(st + (size_t)(hist + r - k) * W + c, v);
+  for (int k = 0; k < CONV_REGT; ++k)
 #pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] += ldf<S>(cw + j * taps + hist - k) * v[j];
+    for (int j = 0; j < V; ++j)
+      wb[k][j] = k <= hist ? ldf<S>(cw + j * taps + hist - k) : 0.f;
+  const int t0 = blockIdx.x * CONV_ROWS;
+  const int t1 = min(T, t0 + CONV_ROWS);
+  for (int t = t0; t < t1; ++t) {
+    const int b = row_seq[t];
+    const int r = t - cu[b];
+    const int p = q_start[b] + r;
+    const float* st = state + (size_t)sslot[b] * (hist > 0 ? hist : 1) * W;
+    float cur[4], acc[4];
+    ldv<float, V>(n + (size_t)t * W + c, cur);
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = cur[j] + wb[0][j] * cur[j];
+#pragma unroll
+    for (int k = 1; k < CONV_REGT; ++k) {
+      if (k > hist || p - k < 0) break;       // before the sequence: zeros
+      float v[4];
+      if (r - k >= 0) ldv<float, V>(n + (size_t)(t - k) * W + c, v);
+      else ldv<float, V>(st + (size_t)(hist + r - k) * W + c, v);
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[j] += wb[k][j] * v[j];
+    }
+    for (int k = CONV_REGT; k <= hist && p - k >= 0; ++k) {
+      float v[4];
+      if (r - k >= 0) ldv<float, V>(n + (size_t)(t - k) * W + c, v);
+      else ldv<float, V>(st + (size_t)(hist + r - k) * W + c, v);
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[j] += ldf<S>(cw + j * taps + hist - k) * v[j];
+    }
+    stv<S, V>(h + (size_t)t * W + c, acc);
   }
-  stv<S, V>(h + (size_t)t * W + c, acc);
 }
 
 // After the convolution: the slot keeps the sequence's last taps-1 inputs.
@@ -446,12 +486,13 @@ AF_EXPORT int afm_canon_conv(void* h, const void* n, const void* w,
   if (taps < 1) return 9003;
   hipStream_t s = (hipStream_t)stream;
   const bool vec = W % 4 == 0 && al16(h) && al16(n) && al16(state);
-  dim3 grid(T, vec ? (W / 4 + 255) / 256 : (W + 255) / 256);
+  dim3 grid((T + CONV_ROWS - 1) / CONV_ROWS,
+            vec ? (W / 4 + 255) / 256 : (W + 255) / 256);
 #define CC(S, V)                                                              \
   canon_conv_kernel<S, V><<<grid, 256, 0, s>>>(                               \
       (S*)h, (const float*)n, (const S*)w, (const float*)state,               \
       (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,               \
-      (const i32*)sslot, W, taps)
+      (const i32*)sslot, T, W, taps)
   if (dt == 0) { if (vec) CC(u16, 4); else CC(u16, 1); }
   else if (dt == 1) { if (vec) CC(float, 4); else CC(float, 1); }
   else return 9002;
