@@ -256,10 +256,15 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
 // case of decode steps when many heads share one K/V head (16 heads on one
 // latent row are exactly one 16-row tile), where a lane-per-key walk spends
 // its time on H dot products per key.  Workgroup = (token, K/V group x block
-// of 64 heads, key split); wave w owns heads 16w..16w+15 of the block and all
-// four waves stage the 64-key tiles.  Key splits cover multiples of 64 keys;
-// with nsplit > 1 unnormalised outputs and (max, sum) go to part_o [T, H,
-// nsplit, dv] / part_ml [T, H, nsplit, 2] for the split merge.
+// of 16 heads, key split); all four waves hold the block's queries.  Per
+// 64-key tile wave w takes keys 16w..16w+15 for Q K^T with its K fragments
+// loaded straight from the pages (a B fragment is 16 contiguous bytes of a
+// key row), the scores meet in a small LDS tile, every wave repeats the
+// (cheap) softmax of the 16 rows, and wave w accumulates a quarter of the
+// value columns of P V against V^T staged in LDS.  No K tile in LDS: three
+// workgroups fit a CU at value sizes up to 256.  Key splits cover multiples
+// of 64 keys; with nsplit > 1 unnormalised outputs and (max, sum) go to
+// part_o [T, H, nsplit, dv] / part_ml [T, H, nsplit, 2] for the split merge.
 template <int DKC, int DVT, bool VEC>
 __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
     u16* __restrict__ out, const u16* __restrict__ q,
@@ -268,18 +273,19 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
     const i32* __restrict__ positions, float scale, int H, int G, int dk,
     int dv, int page, int maxp, int chunk, int window, i64 ldq, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml, AttnExtra ex) {
-  constexpr int KS = DKC * 32 + 8;
-  constexpr int VS = 72;
-  __shared__ u16 k_lds[64 * KS];
+  constexpr int VS = 72;             // V^T / P row stride (64 tokens + pad)
+  constexpr int SS = 68;             // score row stride (floats)
+  constexpr int DVW = DVT / 4;       // value tiles per wave
   __shared__ u16 v_lds[DVT * 16 * VS];
   __shared__ u16 p_lds[4 * 16 * VS];
+  __shared__ float s_lds[16 * SS];
   __shared__ i32 row_lds[64];
 
   const int t = blockIdx.x, sp = blockIdx.z;
-  const int hpg = H / G, nhb = (hpg + 63) / 64;
+  const int hpg = H / G, nhb = (hpg + 15) / 16;
   const int g = blockIdx.y / nhb, hb = blockIdx.y % nhb;
-  const int hbase = g * hpg + hb * 64;
-  const int nrows = min(64, hpg - hb * 64);
+  const int hbase = g * hpg + hb * 16;
+  const int nrows = min(16, hpg - hb * 16);
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pos = positions[t];
   const i32* btr = bt + (size_t)row_seq[t] * maxp;
@@ -291,13 +297,11 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
     lo += sp * per;
     hi = min(pos, lo + per - 1);
   }
-  const int wrow0 = wid * 16;
-  const bool wave_live = wrow0 < nrows;
   if (lo > hi && !(ex.sink && sp == 0)) {
     // an empty split (the grid is sized for the longest reach): mark it and
     // leave before touching queries or pages
-    for (int i = threadIdx.x; i < nrows; i += 256) {
-      const size_t th = (size_t)t * H + hbase + i;
+    if ((int)threadIdx.x < nrows) {
+      const size_t th = (size_t)t * H + hbase + threadIdx.x;
       part_ml[(th * nsplit + sp) * 2] = AF_NEG_INF;
       part_ml[(th * nsplit + sp) * 2 + 1] = 0.f;
     }
@@ -306,17 +310,17 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
 
   s16x8 q_frag[DKC];
   {
-    const int head = hbase + min(wrow0 + (lane & 15), nrows - 1);
+    const int head = hbase + min(lane & 15, nrows - 1);
     const u16* qr = q + (size_t)t * ldq + (size_t)head * dk;
 #pragma unroll
     for (int c = 0; c < DKC; ++c)
       q_frag[c] = load8<VEC>(qr, c * 32 + (lane >> 4) * 8, dk);
   }
   float m[4], l[4], r1v[4], r2v[4];
-  f32x4 o_acc[DVT];
+  f32x4 o_acc[DVW];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int hr = wrow0 + (lane >> 4) * 4 + r;
+    const int hr = (lane >> 4) * 4 + r;
     const int head = hbase + min(hr, nrows - 1);
     const bool sk = ex.sink && sp == 0 && hr < nrows;   // first split only
     m[r] = sk ? ex.sink[head] : AF_NEG_INF;
@@ -325,40 +329,74 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
     r2v[r] = ex.r1 ? ex.r2[head] : 0.f;
   }
 #pragma unroll
-  for (int dt = 0; dt < DVT; ++dt) o_acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int dw = 0; dw < DVW; ++dw) o_acc[dw] = f32x4{0.f, 0.f, 0.f, 0.f};
   u16* pw = p_lds + wid * 16 * VS;
   const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
 
   for (int kv0 = lo; kv0 <= hi; kv0 += 64) {
+    __syncthreads();   // the previous tile's scores, V^T and rows are read
+    if (threadIdx.x < 64) {
+      const int j = kv0 + threadIdx.x;
+      row_lds[threadIdx.x] =
+          j <= hi ? (btr[j / page] * G + g) * page + (j % page) : -1;
+    }
     __syncthreads();
-    stage_kv_tile<DKC, DVT, VEC>(k_lds, v_lds, row_lds, kc, vc, btr, kv0, hi,
-                                 G, g, page, dk, dv, ex.ldv);
-    __syncthreads();
-    if (!wave_live) continue;
-
-    f32x4 s_acc[4];
-#pragma unroll
-    for (int st = 0; st < 4; ++st) {
-      s_acc[st] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const u16* krow = k_lds + (st * 16 + (lane & 15)) * KS + (lane >> 4) * 8;
+    // ---- this wave's 16 keys: K fragments from the pages ----
+    s16x8 kf[DKC];
+    {
+      const int krow = row_lds[wid * 16 + (lane & 15)];
 #pragma unroll
       for (int c = 0; c < DKC; ++c) {
-        const s16x8 kf = *reinterpret_cast<const s16x8*>(krow + c * 32);
-        s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            as_bf16x8(q_frag[c]), as_bf16x8(kf), s_acc[st], 0, 0, 0);
+        kf[c] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (krow >= 0)
+          kf[c] = load8<VEC>(kc + (size_t)krow * dk, c * 32 + (lane >> 4) * 8, dk);
       }
     }
+    // ---- V^T of the whole tile, all threads ----
+    constexpr int VIT = (32 * DVT * 2 + 255) / 256;
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      const int i = it * 256 + threadIdx.x;
+      if (i >= 32 * DVT * 2) break;
+      const int tp = i % 32, e0 = (i / 32) * 8;
+      const int ra = row_lds[tp * 2], rb = row_lds[tp * 2 + 1];
+      s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
+      if (ra >= 0) a = load8<VEC>(vc + (size_t)ra * ex.ldv, e0, dv);
+      if (rb >= 0) c8 = load8<VEC>(vc + (size_t)rb * ex.ldv, e0, dv);
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
+                                ((uint32_t)(unsigned short)c8[jj] << 16);
+        *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
+      }
+    }
+    // ---- scores of the sub-tile, parked in C layout ----
+    {
+      f32x4 sa = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DKC; ++c)
+        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            as_bf16x8(q_frag[c]), as_bf16x8(kf[c]), sa, 0, 0, 0);
+      const int j = kv0 + wid * 16 + (lane & 15);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float sv = sa[r] * scale;
+        if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
+        if (ex.r1) sv -= attn_dist_bias(r1v[r], r2v[r], max(pos - j, 0));
+        s_lds[((lane >> 4) * 4 + r) * SS + wid * 16 + (lane & 15)] =
+            (j <= hi) ? sv : AF_NEG_INF;
+      }
+    }
+    __syncthreads();
+    // ---- softmax of the 16 rows over the tile, the same in every wave ----
+    f32x4 s_acc[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float sr[4];
       float tmax = AF_NEG_INF;
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
-        const int j = kv0 + st * 16 + (lane & 15);
-        float sv = s_acc[st][r] * scale;
-        if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
-        if (ex.r1) sv -= attn_dist_bias(r1v[r], r2v[r], max(pos - j, 0));
-        sr[st] = (j <= hi) ? sv : AF_NEG_INF;
+        sr[st] = s_lds[((lane >> 4) * 4 + r) * SS + st * 16 + (lane & 15)];
         tmax = fmaxf(tmax, sr[st]);
       }
       tmax = group16_max_f32(tmax);
@@ -374,7 +412,7 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
       l[r] = l[r] * corr + group16_sum_f32(psum);
       m[r] = mn;
 #pragma unroll
-      for (int dt = 0; dt < DVT; ++dt) o_acc[dt][r] *= corr;
+      for (int dw = 0; dw < DVW; ++dw) o_acc[dw][r] *= corr;
     }
 #pragma unroll
     for (int st = 0; st < 4; ++st)
@@ -385,38 +423,39 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
     const s16x8 pf0 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + (lane >> 4) * 8);
     const s16x8 pf1 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + 32 + (lane >> 4) * 8);
     __builtin_amdgcn_wave_barrier();
+    // ---- this wave's value columns ----
 #pragma unroll
-    for (int dt = 0; dt < DVT; ++dt) {
+    for (int dw = 0; dw < DVW; ++dw) {
+      const int dt = wid * DVW + dw;
       const u16* vrow = v_lds + (dt * 16 + (lane & 15)) * VS + (lane >> 4) * 8;
       const s16x8 vf0 = *reinterpret_cast<const s16x8*>(vrow);
       const s16x8 vf1 = *reinterpret_cast<const s16x8*>(vrow + 32);
-      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-          as_bf16x8(pf0), as_bf16x8(vf0), o_acc[dt], 0, 0, 0);
-      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-          as_bf16x8(pf1), as_bf16x8(vf1), o_acc[dt], 0, 0, 0);
+      o_acc[dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf0), as_bf16x8(vf0), o_acc[dw], 0, 0, 0);
+      o_acc[dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf1), as_bf16x8(vf1), o_acc[dw], 0, 0, 0);
     }
   }
 
-  if (!wave_live) return;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int hr = wrow0 + (lane >> 4) * 4 + r;
+    const int hr = (lane >> 4) * 4 + r;
     if (hr >= nrows) continue;
     const size_t th = (size_t)t * H + hbase + hr;
     if (nsplit == 1) {
       const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
 #pragma unroll
-      for (int dt = 0; dt < DVT; ++dt) {
-        const int d = dt * 16 + (lane & 15);
-        if (d < dv) out[th * dv + d] = f2bf(o_acc[dt][r] * inv);
+      for (int dw = 0; dw < DVW; ++dw) {
+        const int d = (wid * DVW + dw) * 16 + (lane & 15);
+        if (d < dv) out[th * dv + d] = f2bf(o_acc[dw][r] * inv);
       }
     } else {
 #pragma unroll
-      for (int dt = 0; dt < DVT; ++dt) {
-        const int d = dt * 16 + (lane & 15);
-        if (d < dv) part_o[(th * nsplit + sp) * dv + d] = o_acc[dt][r];
+      for (int dw = 0; dw < DVW; ++dw) {
+        const int d = (wid * DVW + dw) * 16 + (lane & 15);
+        if (d < dv) part_o[(th * nsplit + sp) * dv + d] = o_acc[dw][r];
       }
-      if ((lane & 15) == 0) {
+      if (wid == 0 && (lane & 15) == 0) {
         part_ml[(th * nsplit + sp) * 2] = m[r];
         part_ml[(th * nsplit + sp) * 2 + 1] = l[r];
       }
@@ -487,7 +526,7 @@ AF_EXPORT int afm_attn_heads_mfma(
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
                      cap, ldv};
   const int hpg = H / G;
-  dim3 grid(T, G * ((hpg + 63) / 64), nsplit), blk(256);
+  dim3 grid(T, G * ((hpg + 15) / 16), nsplit), blk(256);
   hipStream_t s = (hipStream_t)stream;
 #define AHM(DKC, DVT, VEC)                                                     \
   attn_heads_mfma_kernel<DKC, DVT, VEC><<<grid, blk, 0, s>>>(                  \

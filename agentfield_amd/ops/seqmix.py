@@ -293,7 +293,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             and dv <= 512):
         # single rows whose many heads share a K/V head: the heads are the
         # rows of the matrix-core tiles; key splits of 64-key multiples
-        wgs = T * G * -(-(H // G) // 64)
+        wgs = T * G * -(-(H // G) // 16)
         nsplit = max(1, min(16, 2048 // max(1, wgs), -(-reach // 64)))
         part_o = part_ml = None
         if nsplit > 1:
