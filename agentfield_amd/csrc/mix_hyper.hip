@@ -61,6 +61,19 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return s;
 }
 
+// the same for NT threads (a multiple of 64, at most 1024), fixed order
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum_f32(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < NT / 64; ++w) s += red[w];
+  __syncthreads();
+  return s;
+}
+
 // ------------------------------------------------------------ embedding
 // x[t, s, :] = table[ids[t]] for every stream s.
 template <typename S>
@@ -98,13 +111,15 @@ struct ConvTail {
   int taps;
 };
 
-template <typename S, int MS, int V>
-__global__ void __launch_bounds__(256) hyper_step_kernel(
+// NT threads per row: 256 when rows are plenty, 1024 for steps of few rows,
+// whose time is the chain of dependent loads of one workgroup's iterations.
+template <typename S, int MS, int V, int NT>
+__global__ void __launch_bounds__(NT) hyper_step_kernel(
     float* __restrict__ x, const S* __restrict__ y, i64 ldy,
     const float* __restrict__ mixm, const float* __restrict__ outv,
     const float* __restrict__ inv, const S* __restrict__ normw, float eps,
     float* __restrict__ n, int ns, int W, int norm_mode, ConvTail ct) {
-  __shared__ float s_mix[MS * MS], s_in[MS], s_out[MS], red[4];
+  __shared__ float s_mix[MS * MS], s_in[MS], s_out[MS], red[NT / 64];
   const int t = blockIdx.x;
   if (threadIdx.x < MS * MS) {
     const int s = threadIdx.x / MS, r = threadIdx.x % MS;
@@ -123,7 +138,7 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
   constexpr int KEEP = 4;
   float held[KEEP][4];
   int it = 0;
-  for (int c = threadIdx.x * V; c < W; c += 256 * V, ++it) {
+  for (int c = threadIdx.x * V; c < W; c += NT * V, ++it) {
     float xs[MS][4];
 #pragma unroll
     for (int s = 0; s < MS; ++s)
@@ -171,11 +186,11 @@ __global__ void __launch_bounds__(256) hyper_step_kernel(
     }
   }
   if (!inv || norm_mode == 0) return;
-  const float rinv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)W + eps);
+  const float rinv = 1.0f / sqrtf(block_sum<NT>(ss, red) / (float)W + eps);
   const int tail_pos = ct.w ? ct.pos[t] : 0;
   const int tail_slot = ct.w ? ct.sslot[t] : 0;
   it = 0;
-  for (int c = threadIdx.x * V; c < W; c += 256 * V, ++it) {
+  for (int c = threadIdx.x * V; c < W; c += NT * V, ++it) {
     float u[4], w4[4];
     if (it >= KEEP) ldv<float, V>(nr + c, u);   // columns this thread wrote
 #pragma unroll
@@ -295,14 +310,14 @@ __global__ void __launch_bounds__(256) canon_state_kernel(
 // One workgroup per row.  The down projection's row holds the latent (first
 // R values) and one rotary key part (rd values); the latent is RMS-normed
 // with a plain weight, the key part rotated, and [latent | key part] goes to
-// the key pages [P, 1, page, R + rd] at `slot`.  The query of head h is put
-// together as [qa[h, t, :R] | rotate(q[t, h, dim:dim+rd])]: qa is the
-// unrotated query already multiplied into latent space.  Rotation pairs
+// the key pages [P, 1, page, R + rd] at `slot`.  The attention query of head
+// h is [q in latent space (R, already in place) | rotate(q[t, h, dim:dim+rd])]:
+// the kernel fills the rotary slices of qf [T, H, R + rd].  Rotation pairs
 // element 2i with 2i+1 for i < rot/2, angle = position * inv_freq[i] in fp32.
 template <typename S>
 __global__ void __launch_bounds__(256) latent_prep_kernel(
     S* __restrict__ qf, S* __restrict__ kc, const S* __restrict__ q, i64 ldq,
-    const S* __restrict__ dkv, i64 lddkv, const S* __restrict__ qa,
+    const S* __restrict__ dkv, i64 lddkv,
     const S* __restrict__ normw, const float* __restrict__ inv_freq,
     const i32* __restrict__ positions, const i64* __restrict__ slots,
     float eps, int T, int H, int dim, int rd, int R, int rot) {
@@ -342,23 +357,17 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(
     }
   }
   const int dq = dim + rd;
-  for (int i = threadIdx.x; i < H * dkc; i += 256) {
-    const int h = i / dkc, e = i % dkc;
-    float v;
-    if (e < R) {
-      v = ldf<S>(qa + ((size_t)h * T + t) * R + e);
-    } else {
-      const int k = e - R;
-      const S* qr = q + (size_t)t * ldq + (size_t)h * dq + dim;
-      v = ldf<S>(qr + k);
-      if (k < rot) {
-        const int pr = k >> 1;
-        const float o = ldf<S>(qr + (k ^ 1));
-        v = (k & 1) ? v * cs[pr] + o * cs[half + pr]
-                    : v * cs[pr] - o * cs[half + pr];
-      }
+  for (int i = threadIdx.x; i < H * rd; i += 256) {
+    const int h = i / rd, k = i % rd;
+    const S* qr = q + (size_t)t * ldq + (size_t)h * dq + dim;
+    float v = ldf<S>(qr + k);
+    if (k < rot) {
+      const int pr = k >> 1;
+      const float o = ldf<S>(qr + (k ^ 1));
+      v = (k & 1) ? v * cs[pr] + o * cs[half + pr]
+                  : v * cs[pr] - o * cs[half + pr];
     }
-    stf<S>(qf + (size_t)t * H * dkc + i, v);
+    stf<S>(qf + ((size_t)t * H + h) * dkc + R + k, v);
   }
 }
 
@@ -433,10 +442,19 @@ static int launch_hyper_step(float* x, const void* y, i64 ldy,
                              ConvTail ct, hipStream_t s) {
   const bool vec = W % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(n) &&
                    al16(y) && al16(normw) && al16(ct.state) && al16(ct.h);
+  // few rows of many columns: one column group per thread
+  const bool wide = T <= 512 && W / (vec ? 4 : 1) > 256;
 #define HS(MS, V)                                                            \
-  hyper_step_kernel<S, MS, V><<<T, 256, 0, s>>>(                             \
-      x, (const S*)y, ldy, mixm, outv, inv, (const S*)normw, eps, n, ns, W,  \
-      norm_mode, ct)
+  do {                                                                       \
+    if (wide)                                                                \
+      hyper_step_kernel<S, MS, V, 1024><<<T, 1024, 0, s>>>(                  \
+          x, (const S*)y, ldy, mixm, outv, inv, (const S*)normw, eps, n, ns, \
+          W, norm_mode, ct);                                                 \
+    else                                                                     \
+      hyper_step_kernel<S, MS, V, 256><<<T, 256, 0, s>>>(                    \
+          x, (const S*)y, ldy, mixm, outv, inv, (const S*)normw, eps, n, ns, \
+          W, norm_mode, ct);                                                 \
+  } while (0)
   if (ns <= 4) { if (vec) HS(4, 4); else HS(4, 1); }
   else if (ns <= 8) { if (vec) HS(8, 4); else HS(8, 1); }
   else { if (vec) HS(16, 4); else HS(16, 1); }
@@ -505,7 +523,7 @@ AF_EXPORT int afm_canon_conv(void* h, const void* n, const void* w,
 }
 
 AF_EXPORT int afm_latent_prep(void* qf, void* kc, const void* q, i64 ldq,
-                              const void* dkv, i64 lddkv, const void* qa,
+                              const void* dkv, i64 lddkv,
                               const void* normw, const void* inv_freq,
                               const void* positions, const void* slots,
                               float eps, int T, int H, int dim, int rd, int R,
@@ -517,12 +535,12 @@ AF_EXPORT int afm_latent_prep(void* qf, void* kc, const void* q, i64 ldq,
   if (dt == 0)
     latent_prep_kernel<u16><<<T, 256, sm, s>>>(
         (u16*)qf, (u16*)kc, (const u16*)q, ldq, (const u16*)dkv, lddkv,
-        (const u16*)qa, (const u16*)normw, (const float*)inv_freq,
+        (const u16*)normw, (const float*)inv_freq,
         (const i32*)positions, (const i64*)slots, eps, T, H, dim, rd, R, rot);
   else if (dt == 1)
     latent_prep_kernel<float><<<T, 256, sm, s>>>(
         (float*)qf, (float*)kc, (const float*)q, ldq, (const float*)dkv, lddkv,
-        (const float*)qa, (const float*)normw, (const float*)inv_freq,
+        (const float*)normw, (const float*)inv_freq,
         (const i32*)positions, (const i64*)slots, eps, T, H, dim, rd, R, rot);
   else
     return 9002;

@@ -248,9 +248,14 @@ class LatentAttention(nn.Module):
         dkv = p[:, self.c0:self.c0 + self.nc]
         g = p[:, self.g0:self.g0 + self.ng]
         qu = q.view(T, s.heads, s.dim + s.rot_dim)[:, :, :s.dim]
-        qa = torch.bmm(qu.transpose(0, 1), self.uk)          # [H, T, R]
-        qf = sm.latent_prep(q, dkv, qa, self.c_norm, self.eps, self.inv_freq,
-                            positions, cache.k[run], md.slots, s.heads, s.dim)
+        # attention queries per head [q in latent space | rotated part]: the
+        # batched GEMM writes the first slices in place, latent_prep the rest
+        qf = torch.empty(T, s.heads * self.nc, dtype=h.dtype, device=h.device)
+        torch.bmm(qu.transpose(0, 1), self.uk,
+                  out=qf.view(T, s.heads, self.nc)[:, :, :s.kv_rank]
+                  .transpose(0, 1))
+        sm.latent_prep(q, dkv, qf, self.c_norm, self.eps, self.inv_freq,
+                       positions, cache.k[run], md.slots, s.heads, s.dim)
         ol = sm.masked_attention(qf, cache.k[run], None, md, positions,
                                  s.scale, s.heads, window=s.window,
                                  sink=self.sink, v_width=s.kv_rank)

@@ -177,7 +177,7 @@ def _mix_sigs() -> dict:
             "afm_hyper_step": [p, p, i64, p, p, p, p, f, p, i, i, i, i, p, p,
                                p, p, i, p, i, p],
             "afm_canon_conv": [p, p, p, p, p, p, p, p, i, i, i, i, i, p],
-            "afm_latent_prep": [p, p, p, i64, p, i64, p, p, p, p, p, f, i, i,
+            "afm_latent_prep": [p, p, p, i64, p, i64, p, p, p, p, f, i, i,
                                 i, i, i, i, i, p],
             "afm_gate_heads": [p, p, p, i64, i, i, i, i, p],
             "afm_relu2": [p, p, i64, i, i, i, p],

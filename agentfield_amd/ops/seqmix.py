@@ -1073,7 +1073,7 @@ def rotate_pairs(x: torch.Tensor, positions: torch.Tensor,
     return out
 
 
-def latent_prep(q: torch.Tensor, dkv: torch.Tensor, qa: torch.Tensor,
+def latent_prep(q: torch.Tensor, dkv: torch.Tensor, qf: torch.Tensor,
                 norm_w: torch.Tensor, eps: float,
                 inv_freq: torch.Tensor | None, positions: torch.Tensor,
                 kcache: torch.Tensor, slots: torch.Tensor, heads: int,
@@ -1083,9 +1083,10 @@ def latent_prep(q: torch.Tensor, dkv: torch.Tensor, qa: torch.Tensor,
     with a plain weight, the key part rotated (interleaved pairs on its first
     2*len(inv_freq) elements), and [latent | key part] is appended to the key
     pages kcache [P, 1, page, R + rd] at `slots`.  q [T, H*(dim + rd)] holds
-    per head [unrotated | rotary part]; qa [H, T, R] is the unrotated part
-    already carried into latent space.  Returns the attention queries
-    [T, H*(R + rd)] = per head [qa | rotated rotary part]."""
+    per head [unrotated | rotary part].  qf [T, H*(R + rd)] are the attention
+    queries, per head [unrotated part carried into latent space | rotated
+    rotary part]: the caller has filled the first R elements of every head,
+    the rotary slices are written here.  Returns qf."""
     T = q.shape[0]
     H = heads
     R = norm_w.numel()
@@ -1105,13 +1106,12 @@ def latent_prep(q: torch.Tensor, dkv: torch.Tensor, qa: torch.Tensor,
         pg = torch.div(slots, page, rounding_mode="floor")
         off = slots - pg * page
         kcache[pg, 0, off] = torch.cat([c, kr], 1).to(kcache.dtype)
-        qf = torch.cat([qa.float().transpose(0, 1), qr], -1)
-        return qf.reshape(T, H * dkc).to(q.dtype)
-    qf = torch.empty(T, H * dkc, dtype=q.dtype, device=q.device)
-    qa = qa.contiguous()
+        qf.view(T, H, dkc)[..., R:] = qr.to(qf.dtype)
+        return qf
+    assert qf.is_contiguous() and qf.shape == (T, H * dkc)
     rc = _L().afm_latent_prep(
         _lib.ptr(qf), _lib.ptr(kcache), _lib.ptr(q), _rowstride(q),
-        _lib.ptr(dkv), _rowstride(dkv), _lib.ptr(qa), _lib.ptr(norm_w),
+        _lib.ptr(dkv), _rowstride(dkv), _lib.ptr(norm_w),
         _lib.ptr(inv_freq), _lib.ptr(positions), _lib.ptr(slots), float(eps),
         T, H, dim, rd, R, rot, _code(q), _lib.cur_stream())
     _lib.check(rc, "afm_latent_prep")

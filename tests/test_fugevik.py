@@ -207,7 +207,7 @@ def test_kernel_groups_present(device):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(1, 16), (3, 30), (4, 64), (7, 33),
-                                   (16, 8)])
+                                   (16, 8), (4, 2048), (2, 1030), (3, 5001)])
 def test_stream_step_alone(device, dtype, shape):
     """Write a sublayer output into the streams and read the next input out:
     both halves apart and fused, against the oracle's loops."""
@@ -270,7 +270,8 @@ def test_input_conv_alone(device, dtype, taps):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(3, 30, 3), (4, 64, 4), (1, 16, 1),
-                                   (7, 33, 5), (2, 8, 2)])
+                                   (7, 33, 5), (2, 8, 2), (4, 2048, 4),
+                                   (2, 1030, 3), (2, 4500, 2)])
 def test_decode_step_fuses_input_conv(device, dtype, shape):
     """Steps of one row per sequence (write, read, norm, convolution, slot
     moved on in one kernel) against the separate ops, from position 0 on."""
@@ -548,9 +549,10 @@ def test_rotation_pairs_neighbours(device):
     q[:, dim + 1] = 1.0
     kc = torch.zeros(10, 1, 8, R + rd, device=device)
     slots = torch.arange(8, 8 + T, dtype=torch.int64, device=device)
-    qa = torch.zeros(H, T, R, device=device)
-    qf = sm.latent_prep(q, dkv, qa, torch.ones(R, device=device), 0.0, inv,
+    qf = torch.full((T, H * (R + rd)), 5.0, device=device)
+    qf = sm.latent_prep(q, dkv, qf, torch.ones(R, device=device), 0.0, inv,
                         pos, kc, slots, H, dim).cpu()
+    assert (qf[:, :R] == 5.0).all()         # the caller's slice is left alone
     rows = kc.view(-1, R + rd)[8:8 + T].cpu()
     for i, p in enumerate(pos.tolist()):
         a0, a1 = p * 1.0, p * 100.0 ** -0.5
