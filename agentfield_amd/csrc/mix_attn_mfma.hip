@@ -517,7 +517,7 @@ AF_EXPORT int afm_attn_heads_mfma(
   if (T == 0) return 0;
   if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
-  if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
+  if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
   const bool vec = (dk % 8 == 0) && (dv % 8 == 0) && (ldq % 8 == 0) &&
                    (ldv % 8 == 0) &&
                    ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&

@@ -404,7 +404,9 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
   }
 }
 
-// One wave per (row, head): merge the nsplit partial softmaxes.
+// One wave per (row, head): merge the nsplit (<= 64) partial softmaxes.
+// Lane s weighs split s once; empty splits (max = -inf) weigh nothing and
+// their partial outputs are never read.
 template <typename S>
 __global__ void __launch_bounds__(256) attn_split_combine_kernel(
     S* __restrict__ out, const float* __restrict__ part_o,
@@ -413,17 +415,20 @@ __global__ void __launch_bounds__(256) attn_split_combine_kernel(
   if (rh >= n_rh) return;
   const int lane = threadIdx.x & 63;
   const float* ml = part_ml + (size_t)rh * nsplit * 2;
-  float m = AF_NEG_INF;
-  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, ml[2 * s]);
-  float l = 0.f;
-  for (int s = 0; s < nsplit; ++s)
-    if (ml[2 * s] > AF_NEG_INF) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
-  for (int d = lane; d < dv; d += 64) {
+  const float ms = lane < nsplit ? ml[2 * lane] : AF_NEG_INF;
+  const float ls = lane < nsplit ? ml[2 * lane + 1] : 0.f;
+  const float m = wave_max_f32(ms);
+  const float w = ms > AF_NEG_INF ? expf(ms - m) : 0.f;
+  const float inv = 1.0f / wave_sum_f32(w * ls);
+  for (int d0 = 0; d0 < dv; d0 += 64) {
+    const int d = d0 + lane;
     float o = 0.f;
-    for (int s = 0; s < nsplit; ++s)
-      if (ml[2 * s] > AF_NEG_INF)
-        o += part_o[((size_t)rh * nsplit + s) * dv + d] * expf(ml[2 * s] - m);
-    stf<S>(out + (size_t)rh * dv + d, o / l);
+    for (int s = 0; s < nsplit; ++s) {
+      const float ws = __shfl(w, s, 64);
+      if (ws > 0.f && d < dv)
+        o += part_o[((size_t)rh * nsplit + s) * dv + d] * ws;
+    }
+    if (d < dv) stf<S>(out + (size_t)rh * dv + d, o * inv);
   }
 }
 
@@ -677,7 +682,7 @@ static int launch_attention(void* out, const void* q, const void* kc,
                        (size_t)gq * dkp) * sizeof(float);
     const bool vec = dk % EPL == 0 && dv % EPL == 0 && ex.ldv % EPL == 0 &&
                      (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0;
-    if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
+    if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
     dim3 grid(T, G, ((hpg + gq - 1) / gq) * nsplit);
 #define ROWS(GQ, VEC)                                                         \
   attn_rows_kernel<S, GQ, VEC><<<grid, 256, sm, s>>>(                         \
@@ -744,6 +749,7 @@ AF_EXPORT int afm_attn_split_combine(void* out, const void* part_o,
                                      const void* part_ml, int n_rh, int nsplit,
                                      int dv, int dt, void* stream) {
   if (n_rh == 0) return 0;
+  if (nsplit < 1 || nsplit > 64) return 9003;
   hipStream_t s = (hipStream_t)stream;
   if (dt == 0)
     attn_split_combine_kernel<u16><<<(n_rh + 3) / 4, 256, 0, s>>>(
