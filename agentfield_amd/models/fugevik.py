@@ -545,11 +545,11 @@ def _bench_config(name, width, ff, n_layers, heads, kv_heads, dim,
             kind, mixer = "latent_attention", LatentAttnSpec(
                 heads=heads, dim=dim, rot_dim=rot_dim, vdim=dim,
                 kv_rank=kv_rank, scale=(dim + rot_dim) ** -0.5,
-                window=window, rot_dims=rot_dim, rot_base=250000.0)
+                window=window, rot_dims=rot_dim, rot_base=500000.0)
         else:
             kind, mixer = "attention", BiasedAttnSpec(
                 heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim,
-                scale=dim ** -0.5, window=window, softcap=30.0,
+                scale=dim ** -0.5, window=window, softcap=50.0,
                 kv_from=i - 1 if i % 4 == 2 else None)
         layers.append(FLayerSpec(kind=kind, mixer=mixer, ff=ff))
     return FugevikConfig(name=name, vocab_size=vocab, width=width,

@@ -95,7 +95,7 @@ def cfg_odd():
     as many K/V heads as query heads."""
     layers = [
         _with_ff(_lat(3, 10, 6, 14, 50, window=33, dims=6, base=123.0), 30),
-        _with_ff(_att(5, 5, 6, 10, window=9, cap=30.0), 26),
+        _with_ff(_att(5, 5, 6, 10, window=9, cap=20.0), 26),
         _with_ff(_att(5, 5, 6, 10, window=64, cap=1.5, kv_from=1), 18),
         _with_ff(_lat(5, 6, 2, 6, 10), None),
     ]
@@ -372,7 +372,7 @@ def test_latent_attention_alone(device, dtype, shape):
     # heads, kv_heads, dim, vdim, window, cap
     (6, 3, 12, 20, 21, 4.0),
     (1, 1, 8, 8, 0, 0.0),
-    (5, 5, 6, 10, 9, 30.0),
+    (5, 5, 6, 10, 9, 20.0),
     (8, 1, 64, 64, 40, 1.5),
     (24, 2, 8, 8, 21, 3.0),            # twelve heads per K/V head
     (4, 2, 40, 136, 64, 2.0)])         # values wider than 128
