@@ -714,7 +714,8 @@ static int launch_attention(void* out, const void* q, const void* kc,
   if (dv <= 64) ATT(1);
   else if (dv <= 128) ATT(2);
   else if (dv <= 256) ATT(4);
-  else ATT(8);
+  else if (dv <= 512) ATT(8);
+  else ATT(16);
 #undef ATT
   return af_last_err();
 }
@@ -726,7 +727,7 @@ AF_EXPORT int afm_masked_attention(
     int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
     const void* r1, const void* r2, i64 ldv, int dt, void* stream) {
   if (T == 0) return 0;
-  if (G <= 0 || H % G || dv > 512 || dk > 1024) return 9003;
+  if (G <= 0 || H % G || dv > 1024 || dk > 2048) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
                      cap, ldv};

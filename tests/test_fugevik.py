@@ -335,6 +335,7 @@ def _run_mixer(mod, layout, h, device, dtype, portions, page=8, decode_from=None
     (3, 10, 6, 14, 50, 33, 4),
     (2, 32, 16, 32, 144, 50, 16),     # wide rows: latent + key part = 160
     (2, 8, 8, 8, 328, 70, 8),         # wider than 320
+    (2, 8, 16, 8, 600, 50, 16),       # wider than any tile kernel
     (5, 6, 2, 6, 10, 7, 0),           # nothing rotates
     (9, 8, 8, 8, 24, 19, 8),          # many heads on the one latent row
     (20, 16, 8, 12, 40, 0, 8),
