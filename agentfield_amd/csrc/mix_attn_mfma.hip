@@ -51,7 +51,7 @@ __device__ __forceinline__ s16x8 load8(const u16* row, int e0, int n) {
 // is done once per key (row_lds[tok] = row index in the pages, -1 for keys
 // past `last`), so the tile's loads depend on nothing but LDS and are issued
 // back to back.
-template <int DKC, int DVT, bool VEC>
+template <int DKC, int DVT, bool VEC, int NT = 256>
 __device__ __forceinline__ void stage_kv_tile(
     u16* k_lds, u16* v_lds, i32* row_lds, const u16* __restrict__ kc,
     const u16* __restrict__ vc, const i32* __restrict__ btr, int kv0, int last,
@@ -64,20 +64,21 @@ __device__ __forceinline__ void stage_kv_tile(
         j <= last ? (btr[j / page] * G + g) * page + (j % page) : -1;
   }
   __syncthreads();
-  constexpr int KIT = (64 * DKC * 4) / 256;
+  constexpr int KIT = (64 * DKC * 4 + NT - 1) / NT;
 #pragma unroll
   for (int it = 0; it < KIT; ++it) {
-    const int i = it * 256 + threadIdx.x;
+    const int i = it * NT + threadIdx.x;
+    if (i >= 64 * DKC * 4) break;
     const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
     const int row = row_lds[tok];
     s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
     if (row >= 0) v8 = load8<VEC>(kc + (size_t)row * dk, e0, dk);
     *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
   }
-  constexpr int VIT = (32 * DVT * 2 + 255) / 256;
+  constexpr int VIT = (32 * DVT * 2 + NT - 1) / NT;
 #pragma unroll
   for (int it = 0; it < VIT; ++it) {
-    const int i = it * 256 + threadIdx.x;
+    const int i = it * NT + threadIdx.x;
     if (i >= 32 * DVT * 2) break;
     const int tp = i % 32, e0 = (i / 32) * 8;
     const int ra = row_lds[tp * 2], rb = row_lds[tp * 2 + 1];
@@ -93,8 +94,11 @@ __device__ __forceinline__ void stage_kv_tile(
   }
 }
 
-template <int DKC, int DVT, bool VEC>
-__global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
+// NH = 2: two query heads of one K/V group per workgroup (eight waves), so a
+// staged tile serves both and one head's LDS / MFMA waits hide behind the
+// other's VALU work.
+template <int DKC, int DVT, bool VEC, int NH>
+__global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
     u16* __restrict__ out, const u16* __restrict__ q,
     const u16* __restrict__ kc, const u16* __restrict__ vc,
     const i32* __restrict__ bt, const i32* __restrict__ cu,
@@ -105,13 +109,14 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
   constexpr int VS = 72;             // V^T / P row stride (64 tokens + pad)
   __shared__ u16 k_lds[64 * KS];
   __shared__ u16 v_lds[DVT * 16 * VS];
-  __shared__ u16 p_lds[4 * 16 * VS];
-  __shared__ float bias_lds[128];    // distance bias of this tile's distances
+  __shared__ u16 p_lds[NH * 4 * 16 * VS];
+  __shared__ float bias_lds[NH * 128];  // distance bias of this tile's distances
   __shared__ i32 row_lds[64];        // page row of every key of the tile
 
-  const int tile = blockIdx.x, h = blockIdx.y;
+  const int hsel = threadIdx.x >> 8;           // which of the NH heads
+  const int tile = blockIdx.x, h = blockIdx.y * NH + hsel;
   const int g = h / (H / G);
-  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wid = (threadIdx.x >> 6) & 3, lane = threadIdx.x & 63;
   const int b = tile_seq[tile];
   const int r0 = cu[b];
   const int len = cu[b + 1] - r0;
@@ -148,19 +153,21 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
   for (int r = 0; r < 4; ++r) { m[r] = m0; l[r] = ex.sink ? 1.f : 0.f; }
 #pragma unroll
   for (int dt = 0; dt < DVT; ++dt) o_acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  u16* pw = p_lds + wid * 16 * VS;
+  u16* pw = p_lds + (hsel * 4 + wid) * 16 * VS;
   const float r1 = ex.r1 ? ex.r1[h] : 0.f, r2 = ex.r1 ? ex.r2[h] : 0.f;
   const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
 
   for (int kv0 = lo; kv0 <= p_last; kv0 += 64) {
     __syncthreads();   // fragment reads of the previous tile are done
-    stage_kv_tile<DKC, DVT, VEC>(k_lds, v_lds, row_lds, kc, vc, btr, kv0,
-                                 p_last, G, g, page, dk, dv, ex.ldv);
+    stage_kv_tile<DKC, DVT, VEC, 256 * NH>(k_lds, v_lds, row_lds, kc, vc, btr,
+                                           kv0, p_last, G, g, page, dk, dv,
+                                           ex.ldv);
     // distance bias for every distance between a row and a key of the tile:
     // entry i is distance i + (p0 - kv0 - 63); keys ahead of a row are masked
-    if (ex.r1 && threadIdx.x < 127) {
-      const int dist = (int)threadIdx.x + p0 - kv0 - 63;
-      bias_lds[threadIdx.x] = dist > 0 ? attn_dist_bias(r1, r2, dist) : 0.f;
+    if (ex.r1 && (threadIdx.x & 255) < 127) {     // each head its own table
+      const int dist = (int)(threadIdx.x & 255) + p0 - kv0 - 63;
+      bias_lds[hsel * 128 + (threadIdx.x & 255)] =
+          dist > 0 ? attn_dist_bias(r1, r2, dist) : 0.f;
     }
     __syncthreads();
     // keys of this tile that any row of the wave may see
@@ -194,7 +201,7 @@ __global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
         const int j = kv0 + st * 16 + (lane & 15);
         float sv = s_acc[st][r] * scale;
         if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
-        if (ex.r1) sv -= bias_lds[(p - p0) - (j - kv0) + 63];
+        if (ex.r1) sv -= bias_lds[hsel * 128 + (p - p0) - (j - kv0) + 63];
         sr[st] = (j <= p && j >= rlo) ? sv : AF_NEG_INF;
         tmax = fmaxf(tmax, sr[st]);
       }
@@ -486,21 +493,25 @@ AF_EXPORT int afm_attn_prefill_mfma(
   if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
                      cap, ldv};
-  dim3 grid(ntiles, H), blk(256);
+  // two heads per workgroup when a K/V group has an even number of them
+  const bool pair = vec && (H / G) % 2 == 0;
   hipStream_t s = (hipStream_t)stream;
-#define APM(DKC, DVT, VEC)                                                     \
-  attn_prefill_mfma_kernel<DKC, DVT, VEC><<<grid, blk, 0, s>>>(                \
+#define APM(DKC, DVT, VEC, NH)                                                 \
+  attn_prefill_mfma_kernel<DKC, DVT, VEC, NH>                                  \
+      <<<dim3(ntiles, H / NH), 256 * NH, 0, s>>>(                              \
       (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,                \
       (const i32*)bt, (const i32*)cu, (const i32*)q_start,                     \
       (const i32*)tile_seq, (const i32*)tile_q0, scale, H, G, dk, dv, page,    \
       maxp, chunk, window, ldq, ex)
   const bool small = dk <= 64 && dv <= 64;
-  if (dk > 320 || dv > 256) APM(18, 32, true);
-  else if (dk > 128 || dv > 128) APM(10, 16, true);
-  else if (small && vec) APM(2, 4, true);
-  else if (small) APM(2, 4, false);
-  else if (vec) APM(4, 8, true);
-  else APM(4, 8, false);
+  if (dk > 320 || dv > 256) APM(18, 32, true, 1);    // LDS holds one head's tiles
+  else if (dk > 128 || dv > 128) { if (pair) APM(10, 16, true, 2); else APM(10, 16, true, 1); }
+  else if (small && pair) APM(2, 4, true, 2);
+  else if (small && vec) APM(2, 4, true, 1);
+  else if (small) APM(2, 4, false, 1);
+  else if (pair) APM(4, 8, true, 2);
+  else if (vec) APM(4, 8, true, 1);
+  else APM(4, 8, false, 1);
 #undef APM
   return af_last_err();
 }
