@@ -46,41 +46,42 @@ __device__ __forceinline__ s16x8 load8(const u16* row, int e0, int n) {
   return v;
 }
 
-// Stage one 64-key tile: K rows row-major into k_lds, V rows transposed into
+// Stage one tile of KT keys: K rows row-major into k_lds, V rows transposed into
 // v_lds ([d][token], token pairs packed into 32-bit writes).  The page walk
 // is done once per key (row_lds[tok] = row index in the pages, -1 for keys
 // past `last`), so the tile's loads depend on nothing but LDS and are issued
 // back to back.
-template <int DKC, int DVT, bool VEC, int NT = 256>
+template <int DKC, int DVT, bool VEC, int NT = 256, int KT = 64>
 __device__ __forceinline__ void stage_kv_tile(
     u16* k_lds, u16* v_lds, i32* row_lds, const u16* __restrict__ kc,
     const u16* __restrict__ vc, const i32* __restrict__ btr, int kv0, int last,
     int G, int g, int page, int dk, int dv, i64 ldv) {
   constexpr int KS = DKC * 32 + 8;
-  constexpr int VS = 72;
-  if (threadIdx.x < 64) {
+  constexpr int VS = KT + 8;
+  constexpr int TP = KT / 2;                  // token pairs
+  if (threadIdx.x < KT) {
     const int j = kv0 + threadIdx.x;
     row_lds[threadIdx.x] =
         j <= last ? (btr[j / page] * G + g) * page + (j % page) : -1;
   }
   __syncthreads();
-  constexpr int KIT = (64 * DKC * 4 + NT - 1) / NT;
+  constexpr int KIT = (KT * DKC * 4 + NT - 1) / NT;
 #pragma unroll
   for (int it = 0; it < KIT; ++it) {
     const int i = it * NT + threadIdx.x;
-    if (i >= 64 * DKC * 4) break;
+    if (i >= KT * DKC * 4) break;
     const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
     const int row = row_lds[tok];
     s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
     if (row >= 0) v8 = load8<VEC>(kc + (size_t)row * dk, e0, dk);
     *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
   }
-  constexpr int VIT = (32 * DVT * 2 + NT - 1) / NT;
+  constexpr int VIT = (TP * DVT * 2 + NT - 1) / NT;
 #pragma unroll
   for (int it = 0; it < VIT; ++it) {
     const int i = it * NT + threadIdx.x;
-    if (i >= 32 * DVT * 2) break;
-    const int tp = i % 32, e0 = (i / 32) * 8;
+    if (i >= TP * DVT * 2) break;
+    const int tp = i % TP, e0 = (i / TP) * 8;
     const int ra = row_lds[tp * 2], rb = row_lds[tp * 2 + 1];
     s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
     if (ra >= 0) a = load8<VEC>(vc + (size_t)ra * ldv, e0, dv);
@@ -96,22 +97,25 @@ __device__ __forceinline__ void stage_kv_tile(
 
 // NH = 2: two query heads of one K/V group per workgroup (eight waves), so a
 // staged tile serves both and one head's LDS / MFMA waits hide behind the
-// other's VALU work.
-template <int DKC, int DVT, bool VEC, int NH>
-__global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
+// other's VALU work.  KT: keys per staged tile (64, or 32 where two heads'
+// 64-key tiles would not fit in LDS).
+template <int DKC, int DVT, bool VEC, int NH, int KT>
+__device__ __forceinline__ void attn_prefill_mfma_body(
     u16* __restrict__ out, const u16* __restrict__ q,
     const u16* __restrict__ kc, const u16* __restrict__ vc,
     const i32* __restrict__ bt, const i32* __restrict__ cu,
     const i32* __restrict__ q_start, const i32* __restrict__ tile_seq,
     const i32* __restrict__ tile_q0, float scale, int H, int G, int dk, int dv,
-    int page, int maxp, int chunk, int window, i64 ldq, AttnExtra ex) {
+    int page, int maxp, int chunk, int window, i64 ldq, const AttnExtra& ex) {
   constexpr int KS = DKC * 32 + 8;   // K row stride in LDS (elements)
-  constexpr int VS = 72;             // V^T / P row stride (64 tokens + pad)
-  __shared__ u16 k_lds[64 * KS];
+  constexpr int VS = KT + 8;         // V^T / P row stride (KT tokens + pad)
+  constexpr int NST = KT / 16;       // 16-key sub-tiles
+  constexpr int NHF = KT / 32;       // 32-key halves of P V
+  __shared__ u16 k_lds[KT * KS];
   __shared__ u16 v_lds[DVT * 16 * VS];
   __shared__ u16 p_lds[NH * 4 * 16 * VS];
   __shared__ float bias_lds[NH * 128];  // distance bias of this tile's distances
-  __shared__ i32 row_lds[64];        // page row of every key of the tile
+  __shared__ i32 row_lds[KT];        // page row of every key of the tile
 
   const int hsel = threadIdx.x >> 8;           // which of the NH heads
   const int tile = blockIdx.x, h = blockIdx.y * NH + hsel;
@@ -157,27 +161,27 @@ __global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
   const float r1 = ex.r1 ? ex.r1[h] : 0.f, r2 = ex.r1 ? ex.r2[h] : 0.f;
   const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
 
-  for (int kv0 = lo; kv0 <= p_last; kv0 += 64) {
+  for (int kv0 = lo; kv0 <= p_last; kv0 += KT) {
     __syncthreads();   // fragment reads of the previous tile are done
-    stage_kv_tile<DKC, DVT, VEC, 256 * NH>(k_lds, v_lds, row_lds, kc, vc, btr,
-                                           kv0, p_last, G, g, page, dk, dv,
-                                           ex.ldv);
+    stage_kv_tile<DKC, DVT, VEC, 256 * NH, KT>(k_lds, v_lds, row_lds, kc, vc,
+                                               btr, kv0, p_last, G, g, page,
+                                               dk, dv, ex.ldv);
     // distance bias for every distance between a row and a key of the tile:
-    // entry i is distance i + (p0 - kv0 - 63); keys ahead of a row are masked
-    if (ex.r1 && (threadIdx.x & 255) < 127) {     // each head its own table
-      const int dist = (int)(threadIdx.x & 255) + p0 - kv0 - 63;
+    // entry i is distance i + (p0 - kv0 - (KT-1)); keys ahead of a row are masked
+    if (ex.r1 && (threadIdx.x & 255) < 63 + KT) {     // each head its own table
+      const int dist = (int)(threadIdx.x & 255) + p0 - kv0 - (KT - 1);
       bias_lds[hsel * 128 + (threadIdx.x & 255)] =
           dist > 0 ? attn_dist_bias(r1, r2, dist) : 0.f;
     }
     __syncthreads();
     // keys of this tile that any row of the wave may see
     if (!wave_live || kv0 > wp_last) continue;
-    if (window > 0 && kv0 + 63 <= wp0 - window) continue;
+    if (window > 0 && kv0 + KT - 1 <= wp0 - window) continue;
 
-    // ---- S = Q K^T: four 16-key sub-tiles ----
-    f32x4 s_acc[4];
+    // ---- S = Q K^T: 16-key sub-tiles ----
+    f32x4 s_acc[NST];
 #pragma unroll
-    for (int st = 0; st < 4; ++st) {
+    for (int st = 0; st < NST; ++st) {
       s_acc[st] = f32x4{0.f, 0.f, 0.f, 0.f};
       const u16* krow = k_lds + (st * 16 + (lane & 15)) * KS + (lane >> 4) * 8;
 #pragma unroll
@@ -194,14 +198,14 @@ __global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
       int rlo = 0;
       if (chunk > 0) rlo = (p / chunk) * chunk;
       if (window > 0) rlo = max(rlo, p - window + 1);
-      float sr[4];
+      float sr[NST];
       float tmax = AF_NEG_INF;
 #pragma unroll
-      for (int st = 0; st < 4; ++st) {
+      for (int st = 0; st < NST; ++st) {
         const int j = kv0 + st * 16 + (lane & 15);
         float sv = s_acc[st][r] * scale;
         if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
-        if (ex.r1) sv -= bias_lds[hsel * 128 + (p - p0) - (j - kv0) + 63];
+        if (ex.r1) sv -= bias_lds[hsel * 128 + (p - p0) - (j - kv0) + KT - 1];
         sr[st] = (j <= p && j >= rlo) ? sv : AF_NEG_INF;
         tmax = fmaxf(tmax, sr[st]);
       }
@@ -210,7 +214,7 @@ __global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
       const float corr = (m[r] <= AF_NEG_INF) ? 0.f : __expf(m[r] - mn);
       float psum = 0.f;
 #pragma unroll
-      for (int st = 0; st < 4; ++st) {
+      for (int st = 0; st < NST; ++st) {
         sr[st] = (sr[st] <= AF_NEG_INF) ? 0.f : __expf(sr[st] - mn);
         psum += sr[st];
         s_acc[st][r] = sr[st];
@@ -222,24 +226,26 @@ __global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
     }
     // ---- P: C layout -> A fragments through the wave's LDS tile ----
 #pragma unroll
-    for (int st = 0; st < 4; ++st)
+    for (int st = 0; st < NST; ++st)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         pw[((lane >> 4) * 4 + r) * VS + st * 16 + (lane & 15)] = f2bf(s_acc[st][r]);
     __builtin_amdgcn_wave_barrier();
-    const s16x8 pf0 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + (lane >> 4) * 8);
-    const s16x8 pf1 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + 32 + (lane >> 4) * 8);
+    s16x8 pf[NHF];
+#pragma unroll
+    for (int hf = 0; hf < NHF; ++hf)
+      pf[hf] = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + hf * 32 + (lane >> 4) * 8);
     __builtin_amdgcn_wave_barrier();
     // ---- O += P V ----
 #pragma unroll
     for (int dt = 0; dt < DVT; ++dt) {
       const u16* vrow = v_lds + (dt * 16 + (lane & 15)) * VS + (lane >> 4) * 8;
-      const s16x8 vf0 = *reinterpret_cast<const s16x8*>(vrow);
-      const s16x8 vf1 = *reinterpret_cast<const s16x8*>(vrow + 32);
-      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-          as_bf16x8(pf0), as_bf16x8(vf0), o_acc[dt], 0, 0, 0);
-      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-          as_bf16x8(pf1), as_bf16x8(vf1), o_acc[dt], 0, 0, 0);
+#pragma unroll
+      for (int hf = 0; hf < NHF; ++hf) {
+        const s16x8 vf = *reinterpret_cast<const s16x8*>(vrow + hf * 32);
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            as_bf16x8(pf[hf]), as_bf16x8(vf), o_acc[dt], 0, 0, 0);
+      }
     }
   }
 
@@ -256,6 +262,30 @@ __global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(
       if (d < dv) op[d] = f2bf(o_acc[dt][r] * inv);
     }
   }
+}
+
+#define AF_APM_PARAMS                                                          \
+    u16* __restrict__ out, const u16* __restrict__ q,                          \
+    const u16* __restrict__ kc, const u16* __restrict__ vc,                    \
+    const i32* __restrict__ bt, const i32* __restrict__ cu,                    \
+    const i32* __restrict__ q_start, const i32* __restrict__ tile_seq,         \
+    const i32* __restrict__ tile_q0, float scale, int H, int G, int dk, int dv,\
+    int page, int maxp, int chunk, int window, i64 ldq, AttnExtra ex
+#define AF_APM_ARGS                                                            \
+    out, q, kc, vc, bt, cu, q_start, tile_seq, tile_q0, scale, H, G, dk, dv,   \
+    page, maxp, chunk, window, ldq, ex
+
+template <int DKC, int DVT, bool VEC, int NH, int KT = 64>
+__global__ void __launch_bounds__(256 * NH) attn_prefill_mfma_kernel(AF_APM_PARAMS) {
+  attn_prefill_mfma_body<DKC, DVT, VEC, NH, KT>(AF_APM_ARGS);
+}
+
+// The widest instance keeps 16 x 512 output accumulators and an 18-fragment
+// query per wave: two waves per SIMD (the eight waves of one workgroup) is all
+// a CU can hold of it, so it may use their full register share.
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+attn_prefill_mfma_wide_pair_kernel(AF_APM_PARAMS) {
+  attn_prefill_mfma_body<18, 32, true, 2, 32>(AF_APM_ARGS);
 }
 
 // ------------------------------------------------ single rows, many heads
@@ -496,15 +526,26 @@ AF_EXPORT int afm_attn_prefill_mfma(
   // two heads per workgroup when a K/V group has an even number of them
   const bool pair = vec && (H / G) % 2 == 0;
   hipStream_t s = (hipStream_t)stream;
-#define APM(DKC, DVT, VEC, NH)                                                 \
-  attn_prefill_mfma_kernel<DKC, DVT, VEC, NH>                                  \
+#define APM(DKC, DVT, VEC, NH, ...)                                            \
+  attn_prefill_mfma_kernel<DKC, DVT, VEC, NH, ##__VA_ARGS__>                   \
       <<<dim3(ntiles, H / NH), 256 * NH, 0, s>>>(                              \
       (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,                \
       (const i32*)bt, (const i32*)cu, (const i32*)q_start,                     \
       (const i32*)tile_seq, (const i32*)tile_q0, scale, H, G, dk, dv, page,    \
       maxp, chunk, window, ldq, ex)
   const bool small = dk <= 64 && dv <= 64;
-  if (dk > 320 || dv > 256) APM(18, 32, true, 1);    // LDS holds one head's tiles
+  // the widest heads pair up over 32-key tiles: two heads' 64-key tiles are
+  // 164 KB of LDS
+  if (dk > 320 || dv > 256) {
+    if (pair)
+      attn_prefill_mfma_wide_pair_kernel<<<dim3(ntiles, H / 2), 512, 0, s>>>(
+          (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,
+          (const i32*)bt, (const i32*)cu, (const i32*)q_start,
+          (const i32*)tile_seq, (const i32*)tile_q0, scale, H, G, dk, dv, page,
+          maxp, chunk, window, ldq, ex);
+    else
+      APM(18, 32, true, 1);
+  }
   else if (dk > 128 || dv > 128) { if (pair) APM(10, 16, true, 2); else APM(10, 16, true, 1); }
   else if (small && pair) APM(2, 4, true, 2);
   else if (small && vec) APM(2, 4, true, 1);
