@@ -47,12 +47,15 @@ HIP_SOURCES = [
 #   ssm     selective state-space scan + sigmoid attention
 #   hyper   multi-stream residual mixing, input convolutions, latent-attention
 #           row steps
+#   delta   gated delta-rule recurrence, per-head q/k norm with rotary
+#           positions, norm after the residual sum
 MIX_GROUPS = {
     "glue": (PKG_DIR / "libafglue.so", ["mix_glue.hip"]),
     "seq": (PKG_DIR / "libafmix.so", ["mix_seq.hip", "mix_attn_mfma.hip"]),
     "ssm": (PKG_DIR / "libafssm.so", ["mix_ssm.hip", "mix_sigattn.hip",
                                        "mix_sigattn_mfma.hip"]),
     "hyper": (PKG_DIR / "libafhyper.so", ["mix_hyper.hip"]),
+    "delta": (PKG_DIR / "libafdelta.so", ["mix_delta.hip"]),
 }
 MIX_SOURCES = [s for _lib, srcs in MIX_GROUPS.values() for s in srcs]
 MIX_LIB = MIX_GROUPS["seq"][0]

@@ -7,6 +7,9 @@
 //   softmax denominator += exp(sink[h])         (sink given: a keyless,
 //                                                valueless, unscaled term)
 //
+// first > 0: the keys j < first stay visible to every later row whatever the
+// chunk or window says (at their true positions).
+//
 // ldv is the row stride of the value pages in elements: dv for pages of
 // their own, dk when the values are the leading dv elements of the key rows
 // (vc == kc; latent attention keeps one row per token).
@@ -19,6 +22,7 @@ struct AttnExtra {
   const float* r2;     // [H] (with r1)
   float cap;           // 0: no soft cap
   i64 ldv;
+  int first;           // 0: no always-visible leading keys
 };
 
 // exact forms (fp32 storage and the row kernels)

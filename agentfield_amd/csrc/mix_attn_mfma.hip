@@ -161,7 +161,13 @@ __device__ __forceinline__ void attn_prefill_mfma_body(
   const float r1 = ex.r1 ? ex.r1[h] : 0.f, r2 = ex.r1 ? ex.r2[h] : 0.f;
   const float inv_cap = ex.cap > 0.f ? 1.0f / ex.cap : 0.f;
 
-  for (int kv0 = lo; kv0 <= p_last; kv0 += KT) {
+  // always-visible leading keys that lie in front of the window are walked
+  // first, in whole tiles from key 0; the window's tiles follow from b0
+  const int nfirst = (ex.first > 0 && lo > 0) ? min(ex.first, lo) : 0;
+  const int a_end = (nfirst + KT - 1) / KT * KT;
+  const int b0 = max(lo, a_end);
+  for (int kv0 = nfirst > 0 ? 0 : lo; kv0 <= p_last;
+       kv0 = (kv0 < a_end && kv0 + KT >= a_end) ? b0 : kv0 + KT) {
     __syncthreads();   // fragment reads of the previous tile are done
     stage_kv_tile<DKC, DVT, VEC, 256 * NH, KT>(k_lds, v_lds, row_lds, kc, vc,
                                                btr, kv0, p_last, G, g, page,
@@ -176,7 +182,7 @@ __device__ __forceinline__ void attn_prefill_mfma_body(
     __syncthreads();
     // keys of this tile that any row of the wave may see
     if (!wave_live || kv0 > wp_last) continue;
-    if (window > 0 && kv0 + KT - 1 <= wp0 - window) continue;
+    if (window > 0 && kv0 + KT - 1 <= wp0 - window && kv0 >= ex.first) continue;
 
     // ---- S = Q K^T: 16-key sub-tiles ----
     f32x4 s_acc[NST];
@@ -206,7 +212,7 @@ __device__ __forceinline__ void attn_prefill_mfma_body(
         float sv = s_acc[st][r] * scale;
         if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
         if (ex.r1) sv -= bias_lds[hsel * 128 + (p - p0) - (j - kv0) + KT - 1];
-        sr[st] = (j <= p && j >= rlo) ? sv : AF_NEG_INF;
+        sr[st] = (j <= p && (j >= rlo || j < ex.first)) ? sv : AF_NEG_INF;
         tmax = fmaxf(tmax, sr[st]);
       }
       tmax = group16_max_f32(tmax);
@@ -510,8 +516,10 @@ AF_EXPORT int afm_attn_prefill_mfma(
     const void* cu, const void* q_start, const void* tile_seq,
     const void* tile_q0, float scale, int ntiles, int H, int G, int dk, int dv,
     int page, int maxp, int chunk, int window, i64 ldq, const void* sink,
-    float cap, const void* r1, const void* r2, i64 ldv, void* stream) {
+    float cap, const void* r1, const void* r2, i64 ldv, int keep_first,
+    void* stream) {
   if (ntiles == 0) return 0;
+  if (keep_first < 0) return 9003;
   if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
   const bool vec = (dk % 8 == 0) && (dv % 8 == 0) && (ldq % 8 == 0) &&
@@ -522,7 +530,7 @@ AF_EXPORT int afm_attn_prefill_mfma(
   // to the row kernel
   if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
-                     cap, ldv};
+                     cap, ldv, keep_first};
   // two heads per workgroup when a K/V group has an even number of them
   const bool pair = vec && (H / G) % 2 == 0;
   hipStream_t s = (hipStream_t)stream;
@@ -565,8 +573,11 @@ AF_EXPORT int afm_attn_heads_mfma(
     const void* row_seq, const void* positions, float scale, int T, int H,
     int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
     int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
-    const void* r1, const void* r2, i64 ldv, void* stream) {
+    const void* r1, const void* r2, i64 ldv, int keep_first, void* stream) {
   if (T == 0) return 0;
+  // the head-tile kernel walks one contiguous key range: rows with
+  // always-visible leading keys go to the row kernel
+  if (keep_first > 0) return 9004;
   if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
@@ -576,7 +587,7 @@ AF_EXPORT int afm_attn_heads_mfma(
                    ((uintptr_t)vc % 16 == 0);
   if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
-                     cap, ldv};
+                     cap, ldv, 0};
   const int hpg = H / G;
   dim3 grid(T, G * ((hpg + 15) / 16), nsplit), blk(256);
   hipStream_t s = (hipStream_t)stream;

@@ -1,0 +1,495 @@
+// Kernels of delta-rule decoders with the norm after the residual sum:
+//
+//   delta_scan          gated delta rule, token by token in fp32, with the
+//                       unit-length q / k, the write strength and the decay
+//                       evaluated on the way in
+//   qk_rope_cache       bias, per-head RMSNorm, partial rotate-half rotary
+//                       positions, K/V page append
+//   postnorm_sum        x <- norm(alpha x + sublayer output); the sublayer
+//                       output may be the mean of two separately normed
+//                       branches
+//   gate_gather         act(z) * rows of a per-token table
+//
+// Storage dtype S is bf16 (raw u16) or fp32; statistics, angles, decays, the
+// recurrent state and the residual are fp32.
+#include "common.h"
+
+namespace {
+
+template <typename S> __device__ __forceinline__ float ldf(const S* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename S> __device__ __forceinline__ void stf(S* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+template <typename S> __device__ __forceinline__ void ld4(const S* p, float (&o)[4]);
+template <> __device__ __forceinline__ void ld4<u16>(const u16* p, float (&o)[4]) {
+  const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = bf2f((u16)v[j]);
+}
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float (&o)[4]) {
+  const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = v[j];
+}
+template <typename S> __device__ __forceinline__ void st4(S* p, const float (&o)[4]);
+template <> __device__ __forceinline__ void st4<u16>(u16* p, const float (&o)[4]) {
+  s16x4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = (short)f2bf(o[j]);
+  *reinterpret_cast<s16x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void st4<float>(float* p, const float (&o)[4]) {
+  *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+}
+template <typename S, int V>
+__device__ __forceinline__ void ldv(const S* p, float (&o)[4]) {
+  if (V == 4) ld4<S>(p, o);
+  else { o[0] = ldf<S>(p); o[1] = o[2] = o[3] = 0.f; }
+}
+template <typename S, int V>
+__device__ __forceinline__ void stv(S* p, const float (&o)[4]) {
+  if (V == 4) st4<S>(p, o);
+  else stf<S>(p, o[0]);
+}
+
+template <int N>
+__device__ __forceinline__ void block_sum(float (&v)[N], float* red) {
+#pragma unroll
+  for (int n = 0; n < N; ++n) v[n] = wave_sum_f32(v[n]);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) red[n * 4 + wave] = v[n];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < N; ++n)
+    v[n] = red[n * 4] + red[n * 4 + 1] + red[n * 4 + 2] + red[n * 4 + 3];
+}
+
+template <typename... P>
+inline bool aligned16(P... p) {
+  return ((((uintptr_t)p) % 16 == 0) && ...);
+}
+
+inline int grid_for(i64 n) {
+  i64 g = (n + 255) / 256;
+  return (int)(g < 1 ? 1 : (g > 8192 ? 8192 : g));
+}
+
+__device__ __forceinline__ float softplus_f32(float z) {
+  return z > 20.f ? z : log1pf(expf(z));
+}
+
+// ------------------------------------------------------------ delta scan
+// Workgroup = (sequence, head, 64 state columns); each of its 4 waves owns
+// 16 columns and is independent of the others after staging.  Lane = (row
+// group rg = lane >> 4, column c = lane & 15); a thread keeps the RP rows
+// rg*RP .. rg*RP+RP-1 of its column in registers (4*RP >= dk, rows past dk
+// stay zero).  Per token, with the decayed column d = g * s:
+//     kd = k . d,  qd = q . d        (partial sums, then 2 cross-lane steps)
+//     u  = beta (v - kd);  s = d + k u;  o = qd + (q . k) u
+// which is S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q with the
+// read-out taken after the write.  Tokens advance in blocks of TB: the four
+// waves stage the block's unit-length q and k (q also times q_scale), q . k,
+// decays, write strengths and value columns into LDS, then each wave walks
+// the block alone.  The order of every sum is fixed, so the state does not
+// depend on where a sequence is cut into chunks.
+constexpr int DS_TB = 16;
+
+template <typename S, int RP, bool CH>
+__global__ void __launch_bounds__(256) delta_scan_kernel(
+    float* __restrict__ out, float* __restrict__ state,
+    const S* __restrict__ q, i64 ldq, const S* __restrict__ k, i64 ldk,
+    const S* __restrict__ v, i64 ldv, const S* __restrict__ beta, i64 ldb,
+    const S* __restrict__ dec, i64 ldd, const float* __restrict__ dec_bias,
+    const float* __restrict__ rate, const i32* __restrict__ cu,
+    const i32* __restrict__ q_start, const i32* __restrict__ sslot, int H,
+    int G, int dk, int dv, float q_scale) {
+  constexpr int RS = RP + 4;              // padded row-group segment
+  constexpr int ROW = 4 * RS;             // one token's k (or q, or g) in LDS
+  __shared__ __attribute__((aligned(16))) float k_s[DS_TB * ROW];
+  __shared__ __attribute__((aligned(16))) float q_s[DS_TB * ROW];
+  __shared__ __attribute__((aligned(16))) float g_s[CH ? DS_TB * ROW : 4];
+  __shared__ float v_s[DS_TB * 64];
+  __shared__ float sc_s[DS_TB * 4];       // per token: beta, q.k, scalar decay
+
+  const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 64;
+  const int r0 = cu[b], r1 = cu[b + 1];
+  if (r1 == r0) return;
+  const int g = h / (H / G);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int rg = lane >> 4;
+  const int col = col0 + wave * 16 + (lane & 15);
+  const bool live = col < dv;
+  float* sp = state + ((size_t)sslot[b] * H + h) * (size_t)dk * dv;
+
+  float s[RP];
+#pragma unroll
+  for (int i = 0; i < RP; ++i) {
+    const int row = rg * RP + i;
+    s[i] = (q_start[b] > 0 && live && row < dk) ? sp[(size_t)row * dv + col] : 0.f;
+  }
+  const float rt = rate[h];
+
+  for (int t0 = r0; t0 < r1; t0 += DS_TB) {
+    const int nb = min(DS_TB, r1 - t0);
+    __syncthreads();                       // the previous block is consumed
+    // ---- stage: wave w takes tokens w, w+4, ... ----
+    for (int tt = wave; tt < nb; tt += 4) {
+      const size_t t = (size_t)(t0 + tt);
+      const S* qr = q + t * ldq + (size_t)g * dk;
+      const S* kr = k + t * ldk + (size_t)g * dk;
+      float sq = 0.f, sk = 0.f, qk = 0.f;
+      for (int d = lane; d < dk; d += 64) {
+        const float a = ldf<S>(qr + d), c = ldf<S>(kr + d);
+        sq += a * a;
+        sk += c * c;
+        qk += a * c;
+      }
+      sq = wave_sum_f32(sq);
+      sk = wave_sum_f32(sk);
+      qk = wave_sum_f32(qk);
+      const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+      for (int d = lane; d < 4 * RP; d += 64) {
+        const int o = tt * ROW + (d / RP) * RS + (d % RP);
+        const bool in = d < dk;
+        q_s[o] = in ? ldf<S>(qr + d) * rq : 0.f;
+        k_s[o] = in ? ldf<S>(kr + d) * rk : 0.f;
+        if (CH) {
+          float gv = 1.f;
+          if (in) {
+            const float z = ldf<S>(dec + t * ldd + (size_t)h * dk + d) +
+                            dec_bias[(size_t)h * dk + d];
+            gv = expf(-rt * softplus_f32(z));
+          }
+          g_s[o] = gv;
+        }
+      }
+      if (lane == 0) {
+        sc_s[tt * 4 + 0] = 1.0f / (1.0f + expf(-ldf<S>(beta + t * ldb + h)));
+        sc_s[tt * 4 + 1] = qk * rq * rk;
+        if (!CH) {
+          const float z = ldf<S>(dec + t * ldd + h) + dec_bias[h];
+          sc_s[tt * 4 + 2] = expf(-rt * softplus_f32(z));
+        }
+      }
+      const int vc = col0 + lane;
+      v_s[tt * 64 + lane] =
+          vc < dv ? ldf<S>(v + t * ldv + (size_t)h * dv + vc) : 0.f;
+    }
+    __syncthreads();
+    // ---- walk the block: every wave on its own 16 columns ----
+    for (int tt = 0; tt < nb; ++tt) {
+      const float* kp = k_s + tt * ROW + rg * RS;
+      const float* qp = q_s + tt * ROW + rg * RS;
+      const float* gp = g_s + tt * ROW + rg * RS;
+      const float bt = sc_s[tt * 4 + 0], qk = sc_s[tt * 4 + 1];
+      const float gsc = CH ? 1.f : sc_s[tt * 4 + 2];
+      float kd = 0.f, qd = 0.f;
+      float kk[RP];
+#pragma unroll
+      for (int i = 0; i < RP; i += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kp + i);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qp + i);
+        f32x4 g4 = f32x4{gsc, gsc, gsc, gsc};
+        if (CH) g4 = *reinterpret_cast<const f32x4*>(gp + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float d = s[i + j] * g4[j];
+          s[i + j] = d;
+          kk[i + j] = k4[j];
+          kd += k4[j] * d;
+          qd += q4[j] * d;
+        }
+      }
+      kd += __shfl_xor(kd, 16, 64);
+      qd += __shfl_xor(qd, 16, 64);
+      kd += __shfl_xor(kd, 32, 64);
+      qd += __shfl_xor(qd, 32, 64);
+      const float u = bt * (v_s[tt * 64 + wave * 16 + (lane & 15)] - kd);
+#pragma unroll
+      for (int i = 0; i < RP; ++i) s[i] += kk[i] * u;
+      if (rg == 0 && live)
+        out[(size_t)(t0 + tt) * ((size_t)H * dv) + (size_t)h * dv + col] = qd + qk * u;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+      const int row = rg * RP + i;
+      if (row < dk) sp[(size_t)row * dv + col] = s[i];
+    }
+  }
+}
+
+// ------------------------------------------------ q/k prep for attention
+// One workgroup per row.  Every q head and k head: + bias, RMSNorm over the
+// head with a weight shared by heads, rotate-half rotary positions on the
+// first `rot` dims (dim i pairs with i + rot/2; angle = position * f_i, the
+// product and its sine / cosine taken in double precision).  q goes to a
+// contiguous [T, H*dk] buffer, k and v (+ bias) to their pages.
+template <typename S>
+__global__ void __launch_bounds__(256) qk_rope_cache_kernel(
+    S* __restrict__ qo, const S* __restrict__ q, i64 ldq,
+    const S* __restrict__ k, i64 ldk, const S* __restrict__ v, i64 ldv,
+    const S* __restrict__ qb, const S* __restrict__ kb,
+    const S* __restrict__ vb, const S* __restrict__ qw,
+    const S* __restrict__ kw, const double* __restrict__ inv_freq, int rot,
+    const i32* __restrict__ positions, S* __restrict__ kc, S* __restrict__ vc,
+    const i64* __restrict__ slots, float eps, int H, int G, int dk, int dv,
+    int page) {
+  extern __shared__ float sm[];
+  const int half = rot / 2;
+  float* cs = sm;                          // [half] cos, [half] sin
+  float* buf = sm + 2 * half;              // [4][dk]
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  for (int i = threadIdx.x; i < half; i += 256) {
+    const double a = (double)pos * inv_freq[i];
+    cs[i] = (float)cos(a);
+    cs[half + i] = (float)sin(a);
+  }
+  __syncthreads();
+  const i64 sl = slots[t];
+  const i64 pg = sl / page, off = sl % page;
+  float* nb = buf + wave * dk;
+  for (int u = wave; u < H + G; u += 4) {
+    const bool isq = u < H;
+    const int hh = isq ? u : u - H;
+    const S* src = isq ? q + (size_t)t * ldq + (size_t)hh * dk
+                       : k + (size_t)t * ldk + (size_t)hh * dk;
+    const S* bias = isq ? qb : kb;
+    const S* w = isq ? qw : kw;
+    float ss = 0.f;
+    for (int d = lane; d < dk; d += 64) {
+      float x = ldf<S>(src + d);
+      if (bias) x += ldf<S>(bias + (size_t)hh * dk + d);
+      nb[d] = x;
+      ss += x * x;
+    }
+    ss = wave_sum_f32(ss);
+    const float r = w ? 1.0f / sqrtf(ss / (float)dk + eps) : 1.0f;
+    __builtin_amdgcn_wave_barrier();
+    for (int d = lane; d < dk; d += 64)
+      nb[d] = nb[d] * r * (w ? ldf<S>(w + d) : 1.0f);
+    __builtin_amdgcn_wave_barrier();
+    S* dst = isq ? qo + ((size_t)t * H + hh) * dk
+                 : kc + (((size_t)pg * G + hh) * page + off) * dk;
+    for (int d = lane; d < dk; d += 64) {
+      float o = nb[d];
+      if (d < half) o = o * cs[d] - nb[d + half] * cs[half + d];
+      else if (d < rot) o = o * cs[d - half] + nb[d - half] * cs[d];
+      if (isq || sl >= 0) stf<S>(dst + d, o);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (sl < 0) return;
+  for (int i = threadIdx.x; i < G * dv; i += 256) {
+    float x = ldf<S>(v + (size_t)t * ldv + i);
+    if (vb) x += ldf<S>(vb + i);
+    stf<S>(vc + (((size_t)pg * G + i / dv) * page + off) * dv + (i % dv), x);
+  }
+}
+
+// --------------------------------------------------------- postnorm sum
+// x <- (alpha x + u) / rms(alpha x + u) * w in place on the fp32 residual,
+// also written as h in the storage dtype.  u = y, or with a second branch
+// u = (y / rms(y) * wy + y2 / rms(y2) * wy2) / 2.
+template <typename S, typename YT, int V>
+__global__ void __launch_bounds__(256) postnorm_sum_kernel(
+    float* __restrict__ x, S* __restrict__ h, const YT* __restrict__ y,
+    i64 ldy, const YT* __restrict__ y2, i64 ldy2, const S* __restrict__ wy,
+    const S* __restrict__ wy2, const S* __restrict__ w, float alpha,
+    float eps, int W) {
+  __shared__ float red[8];
+  const int t = blockIdx.x;
+  float* xr = x + (size_t)t * W;
+  const YT* yr = y + (size_t)t * ldy;
+  const YT* y2r = y2 ? y2 + (size_t)t * ldy2 : nullptr;
+  float r1 = 1.f, r2 = 0.f;
+  if (y2r) {
+    float ss[2] = {0.f, 0.f};
+    for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+      float a[4], b[4];
+      ldv<YT, V>(yr + i, a);
+      ldv<YT, V>(y2r + i, b);
+#pragma unroll
+      for (int j = 0; j < V; ++j) { ss[0] += a[j] * a[j]; ss[1] += b[j] * b[j]; }
+    }
+    block_sum<2>(ss, red);
+    r1 = 0.5f / sqrtf(ss[0] / (float)W + eps);
+    r2 = 0.5f / sqrtf(ss[1] / (float)W + eps);
+  }
+  float sv[1] = {0.f};
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float a[4], xv[4];
+    ldv<YT, V>(yr + i, a);
+    ldv<float, V>(xr + i, xv);
+    if (y2r) {
+      float b[4], wa[4], wb[4];
+      ldv<YT, V>(y2r + i, b);
+      ldv<S, V>(wy + i, wa);
+      ldv<S, V>(wy2 + i, wb);
+#pragma unroll
+      for (int j = 0; j < V; ++j) a[j] = a[j] * r1 * wa[j] + b[j] * r2 * wb[j];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      xv[j] = alpha * xv[j] + a[j];
+      sv[0] += xv[j] * xv[j];
+    }
+    stv<float, V>(xr + i, xv);          // re-read below by the same thread
+  }
+  block_sum<1>(sv, red);
+  const float r = 1.0f / sqrtf(sv[0] / (float)W + eps);
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float xv[4], wv[4];
+    ldv<float, V>(xr + i, xv);
+    ldv<S, V>(w + i, wv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) xv[j] = xv[j] * r * wv[j];
+    stv<float, V>(xr + i, xv);
+    if (h) stv<S, V>(h + (size_t)t * W + i, xv);
+  }
+}
+
+// out[t, c] = gelu_tanh(z[t, c]) * table[ids[t], off + c]
+template <typename S>
+__global__ void __launch_bounds__(256) gate_gather_kernel(
+    S* __restrict__ out, const S* __restrict__ z, i64 ldz,
+    const S* __restrict__ table, i64 ldt, int off,
+    const i32* __restrict__ ids, i64 n, int C) {
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    const i64 t = i / C;
+    const int c = (int)(i % C);
+    const float a = ldf<S>(z + t * ldz + c);
+    const float gl = 0.5f * a * (1.0f + tanhf(0.7978845608028654f *
+                                              (a + 0.044715f * a * a * a)));
+    stf<S>(out + i, gl * ldf<S>(table + (size_t)ids[t] * ldt + off + c));
+  }
+}
+
+}  // namespace
+
+#define MIX_DISPATCH(dt, CALL_BF, CALL_F32) \
+  do {                                      \
+    if ((dt) == 0) { CALL_BF; }             \
+    else if ((dt) == 1) { CALL_F32; }       \
+    else return 9002;                       \
+  } while (0)
+
+AF_EXPORT int afm_delta_scan(
+    void* out, void* state, const void* q, i64 ldq, const void* k, i64 ldk,
+    const void* v, i64 ldv, const void* beta, i64 ldb, const void* dec,
+    i64 ldd, const void* dec_bias, const void* rate, const void* cu,
+    const void* q_start, const void* sslot, int B, int H, int G, int dk,
+    int dv, int per_channel, float q_scale, int dt, void* stream) {
+  if (B == 0) return 0;
+  if (H < 1 || G < 1 || H % G != 0 || dk < 1 || dv < 1) return 9003;
+  if (dk > 256) return 9004;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(B, H, (dv + 63) / 64);
+#define DSK(ST, RPV, CHV)                                                   \
+  delta_scan_kernel<ST, RPV, CHV><<<grid, 256, 0, s>>>((float*)out,         \
+      (float*)state, (const ST*)q, ldq, (const ST*)k, ldk, (const ST*)v,    \
+      ldv, (const ST*)beta, ldb, (const ST*)dec, ldd,                       \
+      (const float*)dec_bias, (const float*)rate, (const i32*)cu,           \
+      (const i32*)q_start, (const i32*)sslot, H, G, dk, dv, q_scale)
+#define DSK_CH(ST, RPV)                              \
+  do {                                               \
+    if (per_channel) DSK(ST, RPV, true);             \
+    else DSK(ST, RPV, false);                        \
+  } while (0)
+#define DSK_RP(ST)                                   \
+  do {                                               \
+    if (dk <= 16) DSK_CH(ST, 4);                     \
+    else if (dk <= 32) DSK_CH(ST, 8);                \
+    else if (dk <= 64) DSK_CH(ST, 16);               \
+    else if (dk <= 128) DSK_CH(ST, 32);              \
+    else DSK_CH(ST, 64);                             \
+  } while (0)
+  MIX_DISPATCH(dt, DSK_RP(u16), DSK_RP(float));
+#undef DSK_RP
+#undef DSK_CH
+#undef DSK
+  return af_last_err();
+}
+
+AF_EXPORT int afm_qk_rope_cache(
+    void* qo, const void* q, i64 ldq, const void* k, i64 ldk, const void* v,
+    i64 ldv, const void* qb, const void* kb, const void* vb, const void* qw,
+    const void* kw, const void* inv_freq, int rot, const void* positions,
+    void* kc, void* vc, const void* slots, float eps, int T, int H, int G,
+    int dk, int dv, int page, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (rot < 0 || rot > dk || rot % 2 != 0) return 9003;
+  const size_t smem = (size_t)(rot + 4 * dk) * sizeof(float);
+  if (smem > 60000) return 9004;
+  hipStream_t s = (hipStream_t)stream;
+#define QRC(ST)                                                              \
+  qk_rope_cache_kernel<ST><<<T, 256, smem, s>>>((ST*)qo, (const ST*)q, ldq,  \
+      (const ST*)k, ldk, (const ST*)v, ldv, (const ST*)qb, (const ST*)kb,    \
+      (const ST*)vb, (const ST*)qw, (const ST*)kw, (const double*)inv_freq,  \
+      rot, (const i32*)positions, (ST*)kc, (ST*)vc, (const i64*)slots, eps,  \
+      H, G, dk, dv, page)
+  MIX_DISPATCH(dt, (QRC(u16)), (QRC(float)));
+#undef QRC
+  return af_last_err();
+}
+
+AF_EXPORT int afm_postnorm_sum(void* x, void* h, const void* y, i64 ldy,
+                               int y_f32, const void* y2, i64 ldy2,
+                               const void* wy, const void* wy2, const void* w,
+                               float alpha, float eps, int T, int W, int dt,
+                               void* stream) {
+  if (T == 0) return 0;
+  if (y2 && (!wy || !wy2)) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  const bool vec = W % 4 == 0 && ldy % 4 == 0 && ldy2 % 4 == 0 &&
+                   aligned16(x, h, y, y2, wy, wy2, w);
+#define PNS(ST, YT)                                                          \
+  do {                                                                       \
+    if (vec)                                                                 \
+      postnorm_sum_kernel<ST, YT, 4><<<T, 256, 0, s>>>((float*)x, (ST*)h,    \
+          (const YT*)y, ldy, (const YT*)y2, ldy2, (const ST*)wy,             \
+          (const ST*)wy2, (const ST*)w, alpha, eps, W);                      \
+    else                                                                     \
+      postnorm_sum_kernel<ST, YT, 1><<<T, 256, 0, s>>>((float*)x, (ST*)h,    \
+          (const YT*)y, ldy, (const YT*)y2, ldy2, (const ST*)wy,             \
+          (const ST*)wy2, (const ST*)w, alpha, eps, W);                      \
+  } while (0)
+  if (dt == 0) {
+    if (y_f32) PNS(u16, float);
+    else PNS(u16, u16);
+  } else if (dt == 1) {
+    PNS(float, float);
+  } else {
+    return 9002;
+  }
+#undef PNS
+  return af_last_err();
+}
+
+AF_EXPORT int afm_gate_gather(void* out, const void* z, i64 ldz,
+                              const void* table, i64 ldt, int off,
+                              const void* ids, int T, int C, int dt,
+                              void* stream) {
+  if (T == 0 || C == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const i64 n = (i64)T * C;
+  const int grid = grid_for(n);
+  MIX_DISPATCH(dt,
+      (gate_gather_kernel<u16><<<grid, 256, 0, s>>>((u16*)out, (const u16*)z,
+          ldz, (const u16*)table, ldt, off, (const i32*)ids, n, C)),
+      (gate_gather_kernel<float><<<grid, 256, 0, s>>>((float*)out,
+          (const float*)z, ldz, (const float*)table, ldt, off,
+          (const i32*)ids, n, C)));
+  return af_last_err();
+}

@@ -73,12 +73,13 @@ __device__ __forceinline__ void block_sum(float (&v)[N], float* red) {
 template <typename S>
 __global__ void __launch_bounds__(256) embed_kernel(
     float* __restrict__ out, const S* __restrict__ table,
-    const i32* __restrict__ ids, const float* __restrict__ add, int W) {
+    const i32* __restrict__ ids, const float* __restrict__ add, float scale,
+    int W) {
   const int t = blockIdx.x;
   const S* src = table + (size_t)ids[t] * W;
   float* dst = out + (size_t)t * W;
   for (int i = threadIdx.x; i < W; i += 256)
-    dst[i] = ldf<S>(src + i) + (add ? add[i] : 0.f);
+    dst[i] = ldf<S>(src + i) * scale + (add ? add[i] : 0.f);
 }
 
 __global__ void __launch_bounds__(256) add_rows_kernel(
@@ -193,8 +194,9 @@ __global__ void __launch_bounds__(256) norm_rows_kernel(
   }
 }
 
-// One wave per (row, head): RMS over dv of fp32 o, * weight, * silu(gate).
-template <typename S, int V>
+// One wave per (row, head): RMS over dv of fp32 o, * weight, * silu(gate)
+// (SIG: * sigmoid(gate)).
+template <typename S, int V, bool SIG>
 __global__ void __launch_bounds__(256) headnorm_gate_kernel(
     S* __restrict__ out, const float* __restrict__ o, const S* __restrict__ g,
     const S* __restrict__ w, float eps, int n_rh, int H, int dv, i64 ldg) {
@@ -220,7 +222,7 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(
     if (w) ldv<S, V>(w + d, wv);
 #pragma unroll
     for (int j = 0; j < V; ++j)
-      r[j] = ov[j] * rs * wv[j] * (gv[j] / (1.0f + expf(-gv[j])));
+      r[j] = ov[j] * rs * wv[j] * ((SIG ? 1.0f : gv[j]) / (1.0f + expf(-gv[j])));
     stv<S, V>(out + ((size_t)t * H + h) * dv + d, r);
   }
 }
@@ -360,7 +362,7 @@ __global__ void __launch_bounds__(256) glu_kernel(
     S* __restrict__ out, i64 ldo, i64 ldo_in, const S* __restrict__ g,
     const S* __restrict__ u, i64 ldi, i64 ldi_in, int rg,
     const S* __restrict__ bg, const S* __restrict__ bu,
-    const float* __restrict__ rw, i64 R, int F) {
+    const float* __restrict__ rw, i64 R, int F, float limit) {
   const int FV = F / V;
   const i64 n = R * FV;
   for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
@@ -378,11 +380,18 @@ __global__ void __launch_bounds__(256) glu_kernel(
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       float av = a[j] + ba[j];
+      float uv = b[j] + bb[j];
       if (ACT == 0) av = av / (1.0f + expf(-av));
       else if (ACT == 1) av = fmaxf(av, 0.f);
-      else av = 0.5f * av * (1.0f + tanhf(0.7978845608028654f *
-                                          (av + 0.044715f * av * av * av)));
-      o[j] = av * (b[j] + bb[j]) * wr;
+      else if (ACT == 2)
+        av = 0.5f * av * (1.0f + tanhf(0.7978845608028654f *
+                                       (av + 0.044715f * av * av * av)));
+      else {   // clamped unit: min(g, L) sigmoid(1.702 g) (clamp(u, -L, L) + 1)
+        av = fminf(av, limit);
+        av = av / (1.0f + expf(-1.702f * av));
+        uv = fminf(fmaxf(uv, -limit), limit) + 1.0f;
+      }
+      o[j] = av * uv * wr;
     }
     stv<S, V>(out + (r / rg) * ldo + (r % rg) * ldo_in + c, o);
   }
@@ -399,15 +408,25 @@ __global__ void __launch_bounds__(256) glu_kernel(
 __global__ void __launch_bounds__(64) moe_route_kernel(
     i32* __restrict__ idx, float* __restrict__ wts, float* __restrict__ wd,
     const float* __restrict__ z, const float* __restrict__ corr, int E,
-    int top, int n_groups, int keep, float scale) {
+    int top, int n_groups, int keep, float scale, int softmax, int renorm) {
   extern __shared__ float sh[];
   float* sig = sh;             // [E]
   float* choice = sh + E;      // [E]
   float* gsc = sh + 2 * E;     // [n_groups]
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (size_t)t * E;
+  float zmax = 0.f, zinv = 1.f;
+  if (softmax) {       // scores are softmax(z) over all experts
+    zmax = -INFINITY;
+    for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, zr[e]);
+    zmax = wave_max_f32(zmax);
+    float zs = 0.f;
+    for (int e = lane; e < E; e += 64) zs += expf(zr[e] - zmax);
+    zinv = 1.0f / wave_sum_f32(zs);
+  }
   for (int e = lane; e < E; e += 64) {
-    const float s = 1.0f / (1.0f + expf(-zr[e]));
+    const float s = softmax ? expf(zr[e] - zmax) * zinv
+                            : 1.0f / (1.0f + expf(-zr[e]));
     sig[e] = s;
     choice[e] = s + (corr ? corr[e] : 0.f);
     if (wd) wd[(size_t)t * E + e] = 0.f;
@@ -458,7 +477,7 @@ __global__ void __launch_bounds__(64) moe_route_kernel(
     }
     __syncthreads();
   }
-  const float inv = scale / (total + 1e-20f);
+  const float inv = renorm ? scale / (total + 1e-20f) : scale;
   for (int r = lane; r < top; r += 64) {
     const float w = wts[(size_t)t * top + r] * inv;
     wts[(size_t)t * top + r] = w;
@@ -504,14 +523,15 @@ inline int grid_for(i64 n) {
   } while (0)
 
 AF_EXPORT int afm_embed(void* out, const void* table, const void* ids,
-                        const void* add, int T, int W, int dt, void* stream) {
+                        const void* add, float scale, int T, int W, int dt,
+                        void* stream) {
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   MIX_DISPATCH(dt,
       (embed_kernel<u16><<<T, 256, 0, s>>>((float*)out, (const u16*)table,
-          (const i32*)ids, (const float*)add, W)),
+          (const i32*)ids, (const float*)add, scale, W)),
       (embed_kernel<float><<<T, 256, 0, s>>>((float*)out, (const float*)table,
-          (const i32*)ids, (const float*)add, W)));
+          (const i32*)ids, (const float*)add, scale, W)));
   return af_last_err();
 }
 
@@ -570,17 +590,22 @@ AF_EXPORT int afm_norm_rows(void* out, const void* x, const void* w,
 
 AF_EXPORT int afm_headnorm_gate(void* out, const void* o, const void* g,
                                 const void* w, float eps, int T, int H, int dv,
-                                i64 ldg, int dt, void* stream) {
+                                i64 ldg, int gate_act, int dt, void* stream) {
   if (T == 0) return 0;
   const int n_rh = T * H;
   const int grid = (n_rh + 3) / 4;
   hipStream_t s = (hipStream_t)stream;
   const bool vec = dv % 4 == 0 && ldg % 4 == 0 && aligned16(out, o, g, w);
-#define HG(ST, V)                                                           \
-  headnorm_gate_kernel<ST, V><<<grid, 256, 0, s>>>((ST*)out, (const float*)o, \
-      (const ST*)g, (const ST*)w, eps, n_rh, H, dv, ldg)
-  if (vec) MIX_DISPATCH(dt, (HG(u16, 4)), (HG(float, 4)));
-  else MIX_DISPATCH(dt, (HG(u16, 1)), (HG(float, 1)));
+#define HG(ST, V, SG)                                                       \
+  headnorm_gate_kernel<ST, V, SG><<<grid, 256, 0, s>>>((ST*)out,            \
+      (const float*)o, (const ST*)g, (const ST*)w, eps, n_rh, H, dv, ldg)
+  if (gate_act == 1) {
+    if (vec) MIX_DISPATCH(dt, (HG(u16, 4, true)), (HG(float, 4, true)));
+    else MIX_DISPATCH(dt, (HG(u16, 1, true)), (HG(float, 1, true)));
+  } else {
+    if (vec) MIX_DISPATCH(dt, (HG(u16, 4, false)), (HG(float, 4, false)));
+    else MIX_DISPATCH(dt, (HG(u16, 1, false)), (HG(float, 1, false)));
+  }
 #undef HG
   return af_last_err();
 }
@@ -672,9 +697,9 @@ AF_EXPORT int afm_norm_residual(void* x, void* h, const void* y, i64 ldy,
 AF_EXPORT int afm_glu(void* out, i64 ldo, i64 ldo_in, const void* g,
                       const void* u, i64 ldi, i64 ldi_in, int rg,
                       const void* bg, const void* bu, const void* rw, i64 R,
-                      int F, int act, int dt, void* stream) {
+                      int F, int act, float limit, int dt, void* stream) {
   if (R == 0 || F == 0) return 0;
-  if (act < 0 || act > 2 || rg < 1) return 9003;
+  if (act < 0 || act > 3 || rg < 1) return 9003;
   hipStream_t s = (hipStream_t)stream;
   const bool vec = F % 4 == 0 && ldo % 4 == 0 && ldo_in % 4 == 0 &&
                    ldi % 4 == 0 && ldi_in % 4 == 0 &&
@@ -685,17 +710,18 @@ AF_EXPORT int afm_glu(void* out, i64 ldo, i64 ldo_in, const void* g,
     if (vec)                                                               \
       glu_kernel<ST, A, 4><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,     \
           (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,      \
-          (const ST*)bu, (const float*)rw, R, F);                          \
+          (const ST*)bu, (const float*)rw, R, F, limit);                          \
     else                                                                   \
       glu_kernel<ST, A, 1><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,     \
           (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,      \
-          (const ST*)bu, (const float*)rw, R, F);                          \
+          (const ST*)bu, (const float*)rw, R, F, limit);                          \
   } while (0)
 #define GLU_ACT(ST)                                   \
   do {                                                \
     if (act == 0) GLU(ST, 0);                         \
     else if (act == 1) GLU(ST, 1);                    \
-    else GLU(ST, 2);                                  \
+    else if (act == 2) GLU(ST, 2);                    \
+    else GLU(ST, 3);                                  \
   } while (0)
   MIX_DISPATCH(dt, GLU_ACT(u16), GLU_ACT(float));
 #undef GLU_ACT
@@ -705,8 +731,8 @@ AF_EXPORT int afm_glu(void* out, i64 ldo, i64 ldo_in, const void* g,
 
 AF_EXPORT int afm_moe_route(void* idx, void* wts, void* wd, const void* z,
                             const void* corr, int T, int E, int top,
-                            int n_groups, int keep, float scale,
-                            void* stream) {
+                            int n_groups, int keep, float scale, int softmax,
+                            int renorm, void* stream) {
   if (T == 0) return 0;
   if (E < 1 || top < 1 || top > E) return 9003;
   if (n_groups > 0 && (E % n_groups != 0 || keep < 1)) return 9003;
@@ -715,7 +741,7 @@ AF_EXPORT int afm_moe_route(void* idx, void* wts, void* wd, const void* z,
   if (sm > 60000) return 9004;
   moe_route_kernel<<<T, 64, sm, (hipStream_t)stream>>>(
       (i32*)idx, (float*)wts, (float*)wd, (const float*)z, (const float*)corr,
-      E, top, n_groups, keep, scale);
+      E, top, n_groups, keep, scale, softmax, renorm);
   return af_last_err();
 }
 

@@ -142,6 +142,10 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+  // always-visible leading keys outside the window sit in front of it in a
+  // virtual key index: [lo - nf, lo) stands for the keys [0, nf)
+  const int nf = ex.first > 0 ? min(ex.first, lo) : 0;
+  const int vsh = lo - nf;
   const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
   for (int d = lane; d < dk; d += 64) qs[d] = ldf<S>(qr + d) * scale;
   float m = AF_NEG_INF, l = 0.f;
@@ -150,10 +154,11 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
   float acc[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
-  for (int j0 = lo; j0 <= pos; j0 += 64) {
-    const int j = j0 + lane;
+  for (int j0 = vsh; j0 <= pos; j0 += 64) {
+    const int jv = j0 + lane;
+    const int j = jv < lo ? jv - vsh : jv;
     float s = AF_NEG_INF;
-    if (j <= pos) {
+    if (jv <= pos) {
       const int pg = btr[j / page];
       const S* kr = kc + (((size_t)pg * G + g) * page + (j % page)) * dk;
       float d0 = 0.f;
@@ -163,7 +168,7 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
     }
     const float mn = fmaxf(m, wave_max_f32(s));
     const float corr = (m <= AF_NEG_INF) ? 0.f : expf(m - mn);
-    const float p = (j <= pos) ? expf(s - mn) : 0.f;
+    const float p = (jv <= pos) ? expf(s - mn) : 0.f;
     l = l * corr + wave_sum_f32(p);
     m = mn;
     __builtin_amdgcn_wave_barrier();
@@ -176,7 +181,7 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
       float a = acc[i] * corr;
       if (d < dv) {
         for (int jj = 0; jj < cnt; ++jj) {
-          const int jk = j0 + jj;
+          const int jk = (j0 + jj) < lo ? j0 + jj - vsh : j0 + jj;
           const int pg = btr[jk / page];
           a += ps[jj] * ldf<S>(vc + (((size_t)pg * G + g) * page + (jk % page)) * ex.ldv + d);
         }
@@ -266,6 +271,11 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+  // always-visible leading keys outside the window sit in front of it in a
+  // virtual key index: [wlo - nf, wlo) stands for the keys [0, nf)
+  const int wlo = lo;
+  const int vsh = lo - (ex.first > 0 ? min(ex.first, lo) : 0);
+  lo = vsh;
   if (nsplit > 1) {   // this workgroup's share of [lo, pos]; may be empty
     const int per = (pos - lo + nsplit) / nsplit;
     lo += sp * per;
@@ -300,7 +310,8 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
     // ---- A: scores, one key per lane ----
     if (tile0 == lo) __syncthreads();          // queries are in LDS
     for (int kidx = threadIdx.x; kidx < nk; kidx += 256) {
-      const int j = tile0 + kidx;
+      const int jv = tile0 + kidx;
+      const int j = jv < wlo ? jv - vsh : jv;
       const S* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
       float sco[GQ];
 #pragma unroll
@@ -359,7 +370,8 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
       float vv[4][EPL];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int j = tile0 + min(kb + u * 4 * kpv + kiv, nk - 1);
+        const int jv = tile0 + min(kb + u * 4 * kpv + kiv, nk - 1);
+        const int j = jv < wlo ? jv - vsh : jv;
         const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * ex.ldv;
         load_slice<S, VEC>(vr, liv * EPL, dv, vv[u]);
       }
@@ -725,12 +737,14 @@ AF_EXPORT int afm_masked_attention(
     const void* row_seq, const void* positions, float scale, int T, int H,
     int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
     int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
-    const void* r1, const void* r2, i64 ldv, int dt, void* stream) {
+    const void* r1, const void* r2, i64 ldv, int keep_first, int dt,
+    void* stream) {
   if (T == 0) return 0;
   if (G <= 0 || H % G || dv > 1024 || dk > 2048) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
+  if (keep_first < 0) return 9003;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
-                     cap, ldv};
+                     cap, ldv, keep_first};
   hipStream_t s = (hipStream_t)stream;
   if (dt == 0)
     return launch_attention<u16>(out, q, kc, vc, bt, row_seq, positions, scale,

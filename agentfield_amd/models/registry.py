@@ -85,8 +85,15 @@ def _load_fugevik(path, device="cpu", dtype=None, **kw):
                         max_position=kw.get("max_position"))
 
 
+def _load_vabedra(path, device="cpu", dtype=None, **kw):
+    from .vabedra import load_vabedra
+    return load_vabedra(path, device=device, dtype=dtype,
+                        max_position=kw.get("max_position"))
+
+
 register_architecture(["LlamaForCausalLM", "MistralForCausalLM",
                        "MixtralForCausalLM"], _load_llama)
 register_architecture("Reperax", _load_reperax)
 register_architecture("Zudisun", _load_zudisun)
 register_architecture("Fugevik", _load_fugevik)
+register_architecture("Vabedra", _load_vabedra)

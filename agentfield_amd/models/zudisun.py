@@ -80,7 +80,10 @@ class RoutedSpec:
     groups: int = 0             # 0: no group limit
     keep: int = 0
     shared_ff: int = 0          # 0: no shared expert
-    act: str = "silu"
+    act: str = "silu"           # "clamped": bounded unit, see ops.glu
+    limit: float = 0.0          # bound of the "clamped" unit
+    score: str = "sigmoid"      # or "softmax" over all experts
+    renorm: bool = True         # weights divided by the chosen scores' sum
 
 
 @dataclass
@@ -307,8 +310,8 @@ class GluMLP(nn.Module):
 
 
 class RoutedExperts(nn.Module):
-    """Mixture of gated experts behind a sigmoid router (ops.moe_route) with
-    an optional shared expert.  All gate/up weights sit in one matrix
+    """Mixture of gated experts behind a sigmoid or softmax router
+    (ops.moe_route) with an optional shared expert.  All gate/up weights sit in one matrix
     [E*2F + 2Fs, W] (expert e: rows e*2F.., gate then up; shared last), all
     down weights in one [W, E*F + Fs].
 
@@ -335,13 +338,16 @@ class RoutedExperts(nn.Module):
         z = sm.matmul(h.float(), self.router)
         static = (not md.is_prefill) or T <= MOE_STATIC_ROWS
         idx, wts, wd = sm.moe_route(z, self.correction, s.top, s.groups,
-                                    s.keep, s.scale, dense=static)
+                                    s.keep, s.scale, dense=static,
+                                    score=s.score, renorm=s.renorm)
         if static:
             gu = sm.matmul(h, self.gate_up)
             act = torch.empty(T, E * F + Fs, dtype=h.dtype, device=h.device)
-            sm.glu(gu, F, s.act, units=E, row_weight=wd, out=act)
+            sm.glu(gu, F, s.act, units=E, row_weight=wd, out=act,
+                   limit=s.limit)
             if Fs > 0:
-                sm.glu(gu[:, E * 2 * F:], Fs, s.act, out=act[:, E * F:])
+                sm.glu(gu[:, E * 2 * F:], Fs, s.act, out=act[:, E * F:],
+                       limit=s.limit)
             return sm.matmul(act, self.down), None
         # (row, choice) pairs in expert order; one host round trip for sizes
         flat = idx.flatten().long()
@@ -358,12 +364,13 @@ class RoutedExperts(nn.Module):
                 continue
             a = sm.glu(sm.matmul(xs[o:o + n],
                                  self.gate_up[e * 2 * F:(e + 1) * 2 * F]),
-                       F, s.act)
+                       F, s.act, limit=s.limit)
             ys[o:o + n] = sm.matmul(a, self.down[:, e * F:(e + 1) * F])
             o += n
         shared = None
         if Fs > 0:
-            a = sm.glu(sm.matmul(h, self.gate_up[E * 2 * F:]), Fs, s.act)
+            a = sm.glu(sm.matmul(h, self.gate_up[E * 2 * F:]), Fs, s.act,
+                       limit=s.limit)
             shared = sm.matmul(a, self.down[:, E * F:])
         return sm.moe_combine(ys, pos, wts, shared), None
 

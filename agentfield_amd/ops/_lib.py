@@ -126,13 +126,13 @@ def _mix_sigs() -> dict:
     p, i, i64, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
     return {
         "glue": {
-            "afm_embed": [p, p, p, p, i, i, i, p],
+            "afm_embed": [p, p, p, p, f, i, i, i, p],
             "afm_add_rows": [p, p, p, i, i, p],
             "afm_dual_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, f,
                                     i, i, i, p],
             "afm_scatter_state": [p, p, p, p, i, i, p],
             "afm_norm_rows": [p, p, p, p, f, i, i, i, i, p],
-            "afm_headnorm_gate": [p, p, p, p, f, i, i, i, i64, i, p],
+            "afm_headnorm_gate": [p, p, p, p, f, i, i, i, i64, i, i, p],
             "afm_polynorm": [p, p, p, f, i, i, i64, i, p],
             "afm_gated_residual": [p, p, f, p, f, p, i64, p, p, p, i64, p,
                                    i, i, i, p],
@@ -140,8 +140,8 @@ def _mix_sigs() -> dict:
             "afm_cast_rows": [p, p, i64, i, p],
             "afm_norm_residual": [p, p, p, i64, i, p, p, f, i, i, i, p],
             "afm_glu": [p, i64, i64, p, p, i64, i64, i, p, p, p, i64, i, i,
-                        i, p],
-            "afm_moe_route": [p, p, p, p, p, i, i, i, i, i, f, p],
+                        f, i, p],
+            "afm_moe_route": [p, p, p, p, p, i, i, i, i, i, f, i, i, p],
             "afm_moe_combine": [p, p, p, p, p, i, i, i, i, p],
         },
         "seq": {
@@ -149,11 +149,13 @@ def _mix_sigs() -> dict:
                                   i, i, i, i64, i64, i64, i, p],
             "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i,
                                      i, i, i, i64, i, p, p, p, f, p, p, i64,
-                                     i, p],
+                                     i, i, p],
             "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i,
-                                      i, i, i, i, i, i64, p, f, p, p, i64, p],
+                                      i, i, i, i, i, i64, p, f, p, p, i64, i,
+                                      p],
             "afm_attn_heads_mfma": [p, p, p, p, p, p, p, f, i, i, i, i, i, i,
-                                    i, i, i, i64, i, p, p, p, f, p, p, i64, p],
+                                    i, i, i, i64, i, p, p, p, f, p, p, i64, i,
+                                    p],
             "afm_attn_split_combine": [p, p, p, i, i, i, i, p],
             "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
                                 i, i, i, i, i, i64, i64, i64, i64, i, p],
@@ -181,6 +183,16 @@ def _mix_sigs() -> dict:
                                 i, i, i, i, i, p],
             "afm_gate_heads": [p, p, p, i64, i, i, i, i, p],
             "afm_relu2": [p, p, i64, i, i, i, p],
+        },
+        "delta": {
+            "afm_delta_scan": [p, p, p, i64, p, i64, p, i64, p, i64, p, i64,
+                               p, p, p, p, p, i, i, i, i, i, i, f, i, p],
+            "afm_qk_rope_cache": [p, p, i64, p, i64, p, i64, p, p, p, p, p,
+                                  p, i, p, p, p, p, f, i, i, i, i, i, i, i,
+                                  p],
+            "afm_postnorm_sum": [p, p, p, i64, i, p, i64, p, p, p, f, f, i,
+                                 i, i, p],
+            "afm_gate_gather": [p, p, i64, p, i64, i, p, i, i, i, p],
         },
     }
 

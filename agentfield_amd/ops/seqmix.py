@@ -59,16 +59,19 @@ def _rowstride(t: torch.Tensor) -> int:
 
 # ------------------------------------------------------------------ embed
 def embed_rows(ids: torch.Tensor, table: torch.Tensor,
-               add: torch.Tensor | None = None) -> torch.Tensor:
-    """x[t] = table[ids[t]] (+ add) as an fp32 residual stream [T, W]."""
+               add: torch.Tensor | None = None,
+               scale: float = 1.0) -> torch.Tensor:
+    """x[t] = table[ids[t]] * scale (+ add) as an fp32 residual stream
+    [T, W]."""
     T = ids.numel()
     W = table.shape[1]
     if not _gpu(table):
-        x = table[ids.long()].float()
+        x = table[ids.long()].float() * scale
         return x + add.float() if add is not None else x
     out = torch.empty(T, W, dtype=torch.float32, device=table.device)
     rc = _L().afm_embed(_lib.ptr(out), _lib.ptr(table), _lib.ptr(ids),
-                        _lib.ptr(add), T, W, _code(table), _lib.cur_stream())
+                        _lib.ptr(add), float(scale), T, W, _code(table),
+                        _lib.cur_stream())
     _lib.check(rc, "afm_embed")
     return out
 
@@ -212,11 +215,13 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
                      window: int = 0, sink: torch.Tensor | None = None,
                      softcap: float = 0.0,
                      log_bias: tuple | None = None,
-                     v_width: int = 0) -> torch.Tensor:
+                     v_width: int = 0, keep_first: int = 0) -> torch.Tensor:
     """Softmax attention of packed rows over the paged cache.  Row at
     position i sees key j iff j <= i, and (chunk > 0) floor(j/chunk) ==
-    floor(i/chunk), and (window > 0) j > i - window.  Positions are absolute
-    in the sequence.  q [T, H*dk] -> [T, H*dv]; scores and softmax in fp32.
+    floor(i/chunk), and (window > 0) j > i - window; with keep_first > 0 the
+    keys j < keep_first stay visible whatever chunk and window say, at their
+    true positions.  Positions are absolute in the sequence.  q [T, H*dk] ->
+    [T, H*dv]; scores and softmax in fp32.
 
     Optional terms, per head h: s = q.k * scale; softcap > 0: s <- softcap *
     tanh(s / softcap); log_bias (r1, r2) [H] fp32 each: s <- s - r1[h] *
@@ -247,6 +252,8 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             if window > 0:
                 lo = max(lo, i - window + 1)
             js = torch.arange(lo, i + 1)
+            if keep_first > 0 and lo > 0:
+                js = torch.cat([torch.arange(min(keep_first, lo)), js])
             pg = bt[rs[t]][js // page]
             kk = kcache[pg, :, js % page].float()      # [n, G, dk]
             vv = vsrc[pg, :, js % page][..., :dv].float()
@@ -266,7 +273,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     lens = getattr(md, "seq_lens", None)
     extra = (_lib.ptr(sink), float(softcap), _lib.ptr(r1), _lib.ptr(r2),
-             int(ldv))
+             int(ldv), int(keep_first))
     if (q.dtype == torch.bfloat16 and lens is not None and dk <= 576
             and dv <= 512 and max(lens) >= MFMA_MIN_ROWS):
         # prompt portions: 64-row tiles on the matrix cores
@@ -288,9 +295,9 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             _lib.check(rc, "afm_attn_prefill_mfma")
             return out
     reach = min(x for x in (chunk, window, md.block_table.shape[1] * page)
-                if x > 0)
+                if x > 0) + keep_first
     if (q.dtype == torch.bfloat16 and H // G >= HEADS_MFMA_MIN and dk <= 576
-            and dv <= 512):
+            and dv <= 512 and keep_first == 0):
         # single rows whose many heads share a K/V head: the heads are the
         # rows of the matrix-core tiles; key splits of 64-key multiples
         wgs = T * G * -(-(H // G) // 16)
@@ -419,9 +426,11 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
 def headnorm_gate(o: torch.Tensor, g: torch.Tensor,
                   weight: torch.Tensor | None, eps: float, heads: int,
-                  out_dtype: torch.dtype) -> torch.Tensor:
+                  out_dtype: torch.dtype,
+                  gate_act: str = "silu") -> torch.Tensor:
     """Per-head RMSNorm of o [T, H*dv] fp32 (optional plain weight [dv]
-    shared by heads) times silu(g); g [T, H*dv] may be a strided view."""
+    shared by heads) times silu(g) (gate_act "sigmoid": times sigmoid(g));
+    g [T, H*dv] may be a strided view."""
     T, HD = o.shape
     dv = HD // heads
     if not _gpu(o):
@@ -430,11 +439,15 @@ def headnorm_gate(o: torch.Tensor, g: torch.Tensor,
         if weight is not None:
             of = of * weight.float()
         gf = g.float()
-        return (of.reshape(T, HD) * gf * torch.sigmoid(gf)).to(out_dtype)
+        gate = torch.sigmoid(gf) if gate_act == "sigmoid" else \
+            gf * torch.sigmoid(gf)
+        return (of.reshape(T, HD) * gate).to(out_dtype)
     out = torch.empty(T, HD, dtype=out_dtype, device=o.device)
     rc = _L().afm_headnorm_gate(_lib.ptr(out), _lib.ptr(o), _lib.ptr(g),
                                 _lib.ptr(weight), float(eps), T, heads, dv,
-                                _rowstride(g), _code(out), _lib.cur_stream())
+                                _rowstride(g),
+                                1 if gate_act == "sigmoid" else 0, _code(out),
+                                _lib.cur_stream())
     _lib.check(rc, "afm_headnorm_gate")
     return out
 
@@ -567,7 +580,7 @@ def norm_residual(x: torch.Tensor, y: torch.Tensor,
     return x if h is None else h
 
 
-GLU_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+GLU_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "clamped": 3}
 
 
 def _act(name: str, a: torch.Tensor) -> torch.Tensor:
@@ -582,12 +595,14 @@ def _act(name: str, a: torch.Tensor) -> torch.Tensor:
 def glu(gu: torch.Tensor, F: int, act: str,
         bias: torch.Tensor | None = None, units: int = 1,
         row_weight: torch.Tensor | None = None,
-        out: torch.Tensor | None = None) -> torch.Tensor:
+        out: torch.Tensor | None = None, limit: float = 0.0) -> torch.Tensor:
     """act(gate + bg) * (up + bu) (* row_weight) for `units` gated units
     laid side by side in every row of gu [T, >= units*2F], unit e being
     [gate_e (F) | up_e (F)].  bias [2F] = [bg | bu] (units == 1 only);
-    row_weight [T, units] fp32.  Writes out [T, >= units*F] (allocated
-    [T, units*F] when not given)."""
+    row_weight [T, units] fp32.  act "clamped" is the bounded unit g' *
+    sigmoid(1.702 g') * (u' + 1) with g' = min(gate, limit), u' = clamp(up,
+    -limit, limit).  Writes out [T, >= units*F] (allocated [T, units*F] when
+    not given)."""
     T = gu.shape[0]
     if out is None:
         out = torch.empty(T, units * F, dtype=gu.dtype, device=gu.device)
@@ -596,7 +611,11 @@ def glu(gu: torch.Tensor, F: int, act: str,
         g, u = v[..., :F], v[..., F:]
         if bias is not None:
             g, u = g + bias[:F].float(), u + bias[F:].float()
-        o = _act(act, g) * u
+        if act == "clamped":
+            g = g.clamp(max=limit)
+            o = g * torch.sigmoid(1.702 * g) * (u.clamp(-limit, limit) + 1.0)
+        else:
+            o = _act(act, g) * u
         if row_weight is not None:
             o = o * row_weight.float().reshape(T, units, 1)
         out[:, :units * F] = o.reshape(T, units * F).to(out.dtype)
@@ -607,26 +626,30 @@ def glu(gu: torch.Tensor, F: int, act: str,
         _rowstride(gu), 2 * F, units,
         _lib.ptr(bias[:F]) if bias is not None else None,
         _lib.ptr(bias[F:]) if bias is not None else None,
-        _lib.ptr(row_weight), T * units, F, GLU_ACTS[act], _code(gu),
-        _lib.cur_stream())
+        _lib.ptr(row_weight), T * units, F, GLU_ACTS[act], float(limit),
+        _code(gu), _lib.cur_stream())
     _lib.check(rc, "afm_glu")
     return out
 
 
 def moe_route(z: torch.Tensor, correction: torch.Tensor | None, top: int,
               n_groups: int = 0, keep: int = 0, scale: float = 1.0,
-              dense: bool = False):
-    """Sigmoid router with score correction and group-limited top-k.
+              dense: bool = False, score: str = "sigmoid",
+              renorm: bool = True):
+    """Router with score correction and group-limited top-k.
 
-    z [T, E] fp32 logits; s = sigmoid(z); choice = s + correction.  With
+    z [T, E] fp32 logits; s = sigmoid(z) (score "softmax": softmax(z) over
+    all experts); choice = s + correction.  With
     n_groups > 0 the experts form equal groups of neighbours, a group scores
     the sum of its two largest choice scores and only experts of the `keep`
     best groups can be chosen.  The `top` largest choice scores win; weights
-    = s / (sum of the chosen s + 1e-20) * scale.  Returns (idx [T, top] i32,
+    = s / (sum of the chosen s + 1e-20) * scale (renorm False: s * scale).
+    Returns (idx [T, top] i32,
     weights [T, top] fp32, dense weights [T, E] fp32 or None)."""
     T, E = z.shape
     if not _gpu(z):
-        s = torch.sigmoid(z.float())
+        s = torch.softmax(z.float(), -1) if score == "softmax" else \
+            torch.sigmoid(z.float())
         choice = s + correction.float() if correction is not None else s.clone()
         if n_groups > 0 and keep < n_groups:
             size = E // n_groups
@@ -637,7 +660,8 @@ def moe_route(z: torch.Tensor, correction: torch.Tensor | None, top: int,
                 ~kept.repeat_interleave(size, dim=1), -math.inf)
         idx = choice.topk(top, -1)[1]
         w = s.gather(1, idx)
-        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale if renorm \
+            else w * scale
         wd = None
         if dense:
             wd = torch.zeros(T, E).scatter_(1, idx, w)
@@ -650,7 +674,8 @@ def moe_route(z: torch.Tensor, correction: torch.Tensor | None, top: int,
     rc = _L().afm_moe_route(_lib.ptr(idx), _lib.ptr(w), _lib.ptr(wd),
                             _lib.ptr(z), _lib.ptr(correction), T, E, top,
                             int(n_groups), int(keep), float(scale),
-                            _lib.cur_stream())
+                            1 if score == "softmax" else 0,
+                            1 if renorm else 0, _lib.cur_stream())
     _lib.check(rc, "afm_moe_route")
     return idx, w, wd
 
@@ -1144,4 +1169,222 @@ def relu2(z: torch.Tensor) -> torch.Tensor:
     rc = _L().afm_relu2(_lib.ptr(out), _lib.ptr(z), _rowstride(z), T, F,
                         _code(z), _lib.cur_stream())
     _lib.check(rc, "afm_relu2")
+    return out
+
+
+# =====================================================================
+# Ops of delta-rule decoders with the norm after the residual sum: gated
+# delta rule over per-sequence fp32 state, per-head q/k norm with partial
+# rotary positions (optionally wavelength-scaled frequencies), sublayer
+# outputs summed into a scaled residual and normed, per-token side tables.
+# =====================================================================
+def scaled_inv_freq(dims: int, base: float,
+                    scaling: dict | None = None) -> torch.Tensor:
+    """Rotary frequencies f_i = base^(-2i/dims), i < dims/2, as float64.
+
+    scaling {factor, low, high, original} rescales by wavelength l = 2 pi /
+    f: l < original/high keeps f; l > original/low gives f / factor; in
+    between, with s = (original/l - low) / (high - low), the blend (1 - s) *
+    f / factor + s * f."""
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            orig, fac = float(scaling["original"]), float(scaling["factor"])
+            lo, hi = float(scaling["low"]), float(scaling["high"])
+            wl = 2.0 * math.pi / f
+            if wl > orig / lo:
+                f = f / fac
+            elif wl >= orig / hi:
+                s = (orig / wl - lo) / (hi - lo)
+                f = (1.0 - s) * f / fac + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float64)
+
+
+def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                  heads: int, kv_heads: int, eps: float,
+                  kcache: torch.Tensor, vcache: torch.Tensor,
+                  slots: torch.Tensor, positions: torch.Tensor,
+                  q_bias: torch.Tensor | None = None,
+                  k_bias: torch.Tensor | None = None,
+                  v_bias: torch.Tensor | None = None,
+                  q_norm: torch.Tensor | None = None,
+                  k_norm: torch.Tensor | None = None,
+                  inv_freq: torch.Tensor | None = None) -> torch.Tensor:
+    """Row steps in front of rotary attention.  q [T, H*dk], k [T, G*dk], v
+    [T, G*dv] (strided views allowed) get their biases; every q and k head
+    is RMS-normed over dk with a plain weight [dk] shared by heads (skipped
+    without one); the first 2*len(inv_freq) dims of each head are rotated,
+    dim i paired with i + len(inv_freq), by the angle position * f_i
+    (inv_freq float64; product, sine and cosine in double precision); k and
+    v are appended to the paged caches at `slots`.  Returns q, contiguous
+    [T, H*dk]."""
+    T = q.shape[0]
+    H, G = heads, kv_heads
+    dk = q.shape[1] // H
+    dv = v.shape[1] // G
+    page = kcache.shape[2]
+    half = inv_freq.numel() if inv_freq is not None else 0
+    if not _gpu(q):
+        qf = q.float()
+        kf = k.float()
+        vf = v.float()
+        if q_bias is not None:
+            qf = qf + q_bias.float()
+        if k_bias is not None:
+            kf = kf + k_bias.float()
+        if v_bias is not None:
+            vf = vf + v_bias.float()
+        qf, kf = qf.reshape(T, H, dk), kf.reshape(T, G, dk)
+        if q_norm is not None:
+            qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) \
+                * q_norm.float()
+        if k_norm is not None:
+            kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) \
+                * k_norm.float()
+        if half:
+            ang = positions.double()[:, None] * inv_freq.double()[None]
+            c, s = ang.cos().float()[:, None], ang.sin().float()[:, None]
+
+            def rot(x):
+                u, w = x[..., :half], x[..., half:2 * half]
+                return torch.cat([u * c - w * s, w * c + u * s,
+                                  x[..., 2 * half:]], -1)
+            qf, kf = rot(qf), rot(kf)
+        pg = torch.div(slots, page, rounding_mode="floor")
+        off = slots - pg * page
+        kcache[pg, :, off] = kf.to(kcache.dtype)
+        vcache[pg, :, off] = vf.reshape(T, G, dv).to(vcache.dtype)
+        return qf.reshape(T, H * dk).to(q.dtype)
+    out = torch.empty(T, H * dk, dtype=q.dtype, device=q.device)
+    rc = _L().afm_qk_rope_cache(
+        _lib.ptr(out), _lib.ptr(q), _rowstride(q), _lib.ptr(k), _rowstride(k),
+        _lib.ptr(v), _rowstride(v), _lib.ptr(q_bias), _lib.ptr(k_bias),
+        _lib.ptr(v_bias), _lib.ptr(q_norm), _lib.ptr(k_norm),
+        _lib.ptr(inv_freq), 2 * half, _lib.ptr(positions), _lib.ptr(kcache),
+        _lib.ptr(vcache), _lib.ptr(slots), float(eps), T, H, G, dk, dv, page,
+        _code(q), _lib.cur_stream())
+    _lib.check(rc, "afm_qk_rope_cache")
+    return out
+
+
+def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+               beta: torch.Tensor, decay: torch.Tensor,
+               decay_bias: torch.Tensor, rate: torch.Tensor,
+               state: torch.Tensor, md, heads: int, kv_heads: int,
+               q_scale: float = 1.0) -> torch.Tensor:
+    """Gated delta rule, token by token in fp32, per head h with its q/k
+    head g = h // (heads / kv_heads) and state S [dk, dv]:
+
+        q' = q_g / sqrt(|q_g|^2 + 1e-6) * q_scale,  k' = k_g / sqrt(|k_g|^2 + 1e-6)
+        a  = exp(-rate[h] * softplus(decay + decay_bias))
+        S <- a * S;  u = sigmoid(beta[h]) * (v_h - S^T k');  S <- S + k' u^T
+        o_h = S^T q'                       (the read-out sees the write)
+
+    q, k [T, G*dk], v [T, H*dv], beta [T, H] logits (strided views allowed).
+    decay [T, H] gives one decay per head (decay_bias [H]); decay [T, H*dk]
+    one per head and key channel, scaling the rows of S (decay_bias [H*dk]).
+    rate, decay_bias fp32.  S lives in `state` [slots, H, dk, dv] fp32: read
+    unless the chunk starts at position 0, written after the chunk's last
+    row.  Returns o [T, H*dv] fp32."""
+    T = q.shape[0]
+    H, G = heads, kv_heads
+    dk = q.shape[1] // G
+    dv = v.shape[1] // H
+    per_channel = dk > 1 and decay.shape[1] == H * dk
+    if decay.shape[1] not in (H, H * dk):
+        raise ValueError("delta_scan: decay must be [T, H] or [T, H*dk]")
+    if not _gpu(q):
+        qf = q.float().reshape(T, G, dk)
+        kf = k.float().reshape(T, G, dk)
+        qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + 1e-6) * q_scale
+        kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)
+        qf = qf.repeat_interleave(H // G, dim=1)
+        kf = kf.repeat_interleave(H // G, dim=1)
+        vf = v.float().reshape(T, H, dv)
+        bt = torch.sigmoid(beta.float())
+        z = torch.nn.functional.softplus(decay.float() + decay_bias.float(),
+                                         threshold=20.0)
+        if per_channel:
+            a = torch.exp(-rate.float()[None, :, None] * z.view(T, H, dk))
+            a = a[..., None]
+        else:
+            a = torch.exp(-rate.float()[None] * z)[..., None, None]
+        out = torch.empty(T, H, dv, dtype=torch.float32)
+        cu, qs, sl = (md.cu_seqlens.tolist(), md.q_start.tolist(),
+                      md.state_slots.tolist())
+        for b in range(len(qs)):
+            if cu[b + 1] == cu[b]:
+                continue
+            S = state[sl[b]].clone() if qs[b] > 0 else torch.zeros(H, dk, dv)
+            for t in range(cu[b], cu[b + 1]):
+                S = a[t] * S
+                u = bt[t][:, None] * (vf[t] - torch.einsum("hkv,hk->hv", S,
+                                                           kf[t]))
+                S = S + kf[t][:, :, None] * u[:, None, :]
+                out[t] = torch.einsum("hkv,hk->hv", S, qf[t])
+            state[sl[b]] = S
+        return out.view(T, H * dv)
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+    B = md.q_start.numel()
+    rc = _L().afm_delta_scan(
+        _lib.ptr(out), _lib.ptr(state), _lib.ptr(q), _rowstride(q),
+        _lib.ptr(k), _rowstride(k), _lib.ptr(v), _rowstride(v),
+        _lib.ptr(beta), _rowstride(beta), _lib.ptr(decay), _rowstride(decay),
+        _lib.ptr(decay_bias), _lib.ptr(rate), _lib.ptr(md.cu_seqlens),
+        _lib.ptr(md.q_start), _lib.ptr(md.state_slots), B, H, G, dk, dv,
+        1 if per_channel else 0, float(q_scale), _code(q), _lib.cur_stream())
+    _lib.check(rc, "afm_delta_scan")
+    return out
+
+
+def postnorm_sum(x: torch.Tensor, y: torch.Tensor, alpha: float,
+                 w: torch.Tensor, eps: float, dtype: torch.dtype,
+                 y2: torch.Tensor | None = None,
+                 wy: torch.Tensor | None = None,
+                 wy2: torch.Tensor | None = None) -> torch.Tensor:
+    """In place on the fp32 residual: x <- (alpha x + u) / rms(alpha x + u)
+    * w, the norm sitting after the sum.  u = y, or with a second branch u =
+    (y / rms(y) * wy + y2 / rms(y2) * wy2) / 2.  y (and y2) [T, W] in the
+    storage dtype or fp32.  Returns the new residual in `dtype` (x itself for
+    fp32), the next sublayer's input."""
+    T, W = x.shape
+    if not _gpu(x):
+        def n(u, wt):
+            return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) \
+                * wt.float()
+        u = y.float()
+        if y2 is not None:
+            u = 0.5 * (n(u, wy) + n(y2.float(), wy2))
+        x.copy_(n(alpha * x + u, w))
+        return x.to(dtype) if dtype != torch.float32 else x
+    h = None if dtype == torch.float32 else \
+        torch.empty(T, W, dtype=dtype, device=x.device)
+    if y2 is not None and y2.dtype != y.dtype:
+        raise TypeError("postnorm_sum: both branches in one dtype")
+    rc = _L().afm_postnorm_sum(
+        _lib.ptr(x), _lib.ptr(h), _lib.ptr(y), _rowstride(y),
+        1 if y.dtype == torch.float32 else 0, _lib.ptr(y2),
+        _rowstride(y2) if y2 is not None else 0, _lib.ptr(wy), _lib.ptr(wy2),
+        _lib.ptr(w), float(alpha), float(eps), T, W, _code(w),
+        _lib.cur_stream())
+    _lib.check(rc, "afm_postnorm_sum")
+    return x if h is None else h
+
+
+def gate_gather(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor,
+                offset: int) -> torch.Tensor:
+    """out[t, c] = gelu_tanh(z[t, c]) * table[ids[t], offset + c]: a gate
+    on a slice of a per-token table row.  z [T, C] may be a strided view."""
+    T, C = z.shape
+    if not _gpu(z):
+        e = table[ids.long()][:, offset:offset + C].float()
+        return (_act("gelu_tanh", z.float()) * e).to(z.dtype)
+    out = torch.empty(T, C, dtype=z.dtype, device=z.device)
+    rc = _L().afm_gate_gather(_lib.ptr(out), _lib.ptr(z), _rowstride(z),
+                              _lib.ptr(table), table.stride(0), int(offset),
+                              _lib.ptr(ids), T, C, _code(z),
+                              _lib.cur_stream())
+    _lib.check(rc, "afm_gate_gather")
     return out
