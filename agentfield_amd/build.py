@@ -47,6 +47,7 @@ HIP_SOURCES = [
 #   ssm     selective state-space scan + sigmoid attention
 #   hyper   multi-stream residual mixing, input convolutions, latent-attention
 #           row steps
+#   conv    short depthwise causal convolution with carried inputs
 #   delta   gated delta-rule recurrence, per-head q/k norm with rotary
 #           positions, norm after the residual sum
 MIX_GROUPS = {
@@ -56,6 +57,7 @@ MIX_GROUPS = {
                                        "mix_sigattn_mfma.hip"]),
     "hyper": (PKG_DIR / "libafhyper.so", ["mix_hyper.hip"]),
     "delta": (PKG_DIR / "libafdelta.so", ["mix_delta.hip"]),
+    "conv": (PKG_DIR / "libafconv.so", ["mix_conv.hip"]),
 }
 MIX_SOURCES = [s for _lib, srcs in MIX_GROUPS.values() for s in srcs]
 MIX_LIB = MIX_GROUPS["seq"][0]

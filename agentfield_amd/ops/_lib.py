@@ -160,9 +160,11 @@ def _mix_sigs() -> dict:
             "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
                                 i, i, i, i, i, i64, i64, i64, i64, i, p],
         },
-        "ssm": {
+        "conv": {
             "afm_causal_conv": [p, p, i64, p, p, p, p, p, p, p, i, i, i, i, i,
                                 i, p],
+        },
+        "ssm": {
             "afm_selective_scan": [p, p, p, p, p, p, i64, p, i64, p, p, p, p,
                                    p, i, i, i, i, p],
             "afm_qk_unit_cache": [p, p, i64, p, i64, p, i64, p, i64, f, p, p,

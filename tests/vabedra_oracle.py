@@ -138,19 +138,45 @@ def scaled_frequencies(rot):
     return torch.tensor(out, dtype=F64)
 
 
-def rotate_half(x, rot):
+def rotate_half(x, rot, positions=None):
     """Rotary positions on the first rot.dims elements of each head of
-    x [T, H, d]: element i pairs with i + dims/2."""
+    x [T, H, d]: element i pairs with i + dims/2 (positions 0..T-1 unless
+    given)."""
     if not rot or rot["dims"] == 0:
         return x
     T = x.shape[0]
     half = rot["dims"] // 2
-    ang = torch.arange(T, dtype=F64)[:, None] * scaled_frequencies(rot)[None]
+    pos = torch.arange(T, dtype=F64) if positions is None else \
+        torch.as_tensor(positions, dtype=F64)
+    ang = pos[:, None] * scaled_frequencies(rot)[None]
     c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
     u, w = x[..., :half], x[..., half:2 * half]
     out = x.clone()
     out[..., :half] = u * c - w * s
     out[..., half:2 * half] = w * c + u * s
+    return out
+
+
+def attend(q, k, v, m):
+    """Softmax attention of q [T, H, d] over k [T, G, d], v [T, G, dv], query
+    i seeing key j iff j <= i and (i - j < mask.size or j < mask.keep_first);
+    score q.k * scale, soft-capped; one added to the softmax denominator."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    mask = m.get("mask") or {}
+    size, first = mask.get("size", 0), mask.get("keep_first", 0)
+    cap = m.get("softcap") or 0.0
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for hh in range(H):
+        g = hh // (H // G)
+        for i in range(T):
+            js = [j for j in range(i + 1)
+                  if size <= 0 or i - j < size or j < first]
+            s = (k[js, g] @ q[i, hh]) * m["scale"]
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            e = torch.exp(s)
+            out[i, hh] = (e @ v[js, g]) / (1.0 + e.sum())
     return out
 
 
@@ -162,26 +188,7 @@ def sink_attention(h, P, pre, m, eps):
     v = lin(h, P, pre + "v", True).view(T, G, dv)
     q = rotate_half(rms_norm(q, P[pre + "q.norm"], eps), m.get("rot"))
     k = rotate_half(rms_norm(k, P[pre + "k.norm"], eps), m.get("rot"))
-    mask = m.get("mask") or {}
-    size, first = mask.get("size", 0), mask.get("keep_first", 0)
-    cap = m.get("softcap") or 0.0
-    out = torch.zeros(T, H, dv, dtype=F64)
-    for hh in range(H):
-        g = hh // (H // G)
-        for i in range(T):
-            num = torch.zeros(dv, dtype=F64)
-            den = 1.0                       # the sink: score 0, no value
-            for j in range(i + 1):
-                if size > 0 and i - j >= size and j >= first:
-                    continue
-                s = float(q[i, hh] @ k[j, g]) * m["scale"]
-                if cap > 0:
-                    s = cap * math.tanh(s / cap)
-                e = math.exp(s)
-                den += e
-                num += e * v[j, g]
-            out[i, hh] = num / den
-    return lin(out.reshape(T, H * dv), P, pre + "o")
+    return lin(attend(q, k, v, m).reshape(T, H * dv), P, pre + "o")
 
 
 def parallel_mixer(h, P, pre, m, eps):
@@ -316,7 +323,7 @@ def random_weights(cfg, seed=0):
                 rnd(f"{pre}mlp.e{e}.gate", F, W, std=2.0 * W ** -0.5)
                 rnd(f"{pre}mlp.e{e}.up", F, W, std=2.0 * W ** -0.5)
                 rnd(f"{pre}mlp.e{e}.down", W, F)
-            rnd(pre + "mlp.router", E, W, std=1.5 * W ** -0.5)
+            rnd(pre + "mlp.router", E, W, std=4.0 * W ** -0.5)
             rnd(pre + "mlp.correction", E, std=0.05)
         if side:
             rnd(pre + "side.gate", side, W)
