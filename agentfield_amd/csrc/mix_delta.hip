@@ -81,27 +81,65 @@ inline int grid_for(i64 n) {
   return (int)(g < 1 ? 1 : (g > 8192 ? 8192 : g));
 }
 
-__device__ __forceinline__ float softplus_f32(float z) {
+// exp / softplus / sigmoid on the way into the recurrence.  fp32 storage:
+// the library forms.  bf16 storage: hardware exponential and logarithm (the
+// inputs already carry 2^-9 rounding); softplus switches to e^z below -8 so
+// that 1 + e^z does not swallow it.
+template <typename S> __device__ __forceinline__ float exp_s(float v);
+template <> __device__ __forceinline__ float exp_s<u16>(float v) { return __expf(v); }
+template <> __device__ __forceinline__ float exp_s<float>(float v) { return expf(v); }
+template <typename S> __device__ __forceinline__ float softplus_s(float z);
+template <> __device__ __forceinline__ float softplus_s<u16>(float z) {
+  const float e = __expf(z);
+  return z > 20.f ? z : (z < -8.f ? e : __logf(1.0f + e));
+}
+template <> __device__ __forceinline__ float softplus_s<float>(float z) {
   return z > 20.f ? z : log1pf(expf(z));
+}
+
+template <typename S, int N, bool VEC>
+__device__ __forceinline__ void load_run(const S* p, int e0, int n, float (&o)[N]) {
+  // N consecutive elements from p + e0, zero past n
+  if constexpr (VEC && N >= 4) {
+#pragma unroll
+    for (int j = 0; j < N; j += 4) {
+      float t[4] = {0.f, 0.f, 0.f, 0.f};
+      if (e0 + j < n) ld4<S>(p + e0 + j, t);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[j + i] = t[i];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) o[j] = (e0 + j < n) ? ldf<S>(p + e0 + j) : 0.f;
+  }
+}
+
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __shfl_xor(v, 1, 64);
+  v += __shfl_xor(v, 2, 64);
+  v += __shfl_xor(v, 4, 64);
+  v += __shfl_xor(v, 8, 64);
+  return v;
 }
 
 // ------------------------------------------------------------ delta scan
 // Workgroup = (sequence, head, 64 state columns); each of its 4 waves owns
-// 16 columns and is independent of the others after staging.  Lane = (row
+// 16 columns and walks alone between the staging barriers.  Lane = (row
 // group rg = lane >> 4, column c = lane & 15); a thread keeps the RP rows
 // rg*RP .. rg*RP+RP-1 of its column in registers (4*RP >= dk, rows past dk
 // stay zero).  Per token, with the decayed column d = g * s:
 //     kd = k . d,  qd = q . d        (partial sums, then 2 cross-lane steps)
 //     u  = beta (v - kd);  s = d + k u;  o = qd + (q . k) u
 // which is S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q with the
-// read-out taken after the write.  Tokens advance in blocks of TB: the four
-// waves stage the block's unit-length q and k (q also times q_scale), q . k,
-// decays, write strengths and value columns into LDS, then each wave walks
-// the block alone.  The order of every sum is fixed, so the state does not
-// depend on where a sequence is cut into chunks.
+// read-out taken after the write.  Tokens advance in blocks of 16: sixteen
+// lanes per token fetch the block's q, k, decay logits and values into
+// registers while the previous block is being walked; after the walk they
+// turn them into unit-length q and k (q also times q_scale), q . k, decays
+// and write strengths in LDS.  The order of every sum is fixed, so the state
+// does not depend on where a sequence is cut into chunks.
 constexpr int DS_TB = 16;
 
-template <typename S, int RP, bool CH>
+template <typename S, int RP, bool CH, bool VEC>
 __global__ void __launch_bounds__(256) delta_scan_kernel(
     float* __restrict__ out, float* __restrict__ state,
     const S* __restrict__ q, i64 ldq, const S* __restrict__ k, i64 ldk,
@@ -112,10 +150,11 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
     int G, int dk, int dv, float q_scale) {
   constexpr int RS = RP + 4;              // padded row-group segment
   constexpr int ROW = 4 * RS;             // one token's k (or q, or g) in LDS
+  constexpr int EL = RP / 4;              // staged elements per lane
   __shared__ __attribute__((aligned(16))) float k_s[DS_TB * ROW];
   __shared__ __attribute__((aligned(16))) float q_s[DS_TB * ROW];
   __shared__ __attribute__((aligned(16))) float g_s[CH ? DS_TB * ROW : 4];
-  __shared__ float v_s[DS_TB * 64];
+  __shared__ __attribute__((aligned(16))) float v_s[DS_TB * 64];
   __shared__ float sc_s[DS_TB * 4];       // per token: beta, q.k, scalar decay
 
   const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 64;
@@ -136,53 +175,68 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
   }
   const float rt = rate[h];
 
+  // staging role: token st of the block, elements e0 .. e0 + EL - 1
+  const int st = threadIdx.x >> 4, sub = threadIdx.x & 15;
+  const int e0 = sub * EL;
+  float bias_r[CH ? EL : 1];
+  if (CH) {
+#pragma unroll
+    for (int j = 0; j < EL; ++j)
+      bias_r[j] = e0 + j < dk ? dec_bias[(size_t)h * dk + e0 + j] : 0.f;
+  } else {
+    bias_r[0] = dec_bias[h];
+  }
+  float fq[EL], fk[EL], fz[CH ? EL : 1], fv[4], fb = 0.f;
+  auto fetch = [&](int t0) {
+    const int tt = t0 + st;
+    if (tt < r1) {
+      const size_t t = (size_t)tt;
+      load_run<S, EL, VEC>(q + t * ldq + (size_t)g * dk, e0, dk, fq);
+      load_run<S, EL, VEC>(k + t * ldk + (size_t)g * dk, e0, dk, fk);
+      if (CH) load_run<S, CH ? EL : 1, VEC>(dec + t * ldd + (size_t)h * dk, e0, dk, fz);
+      else fz[0] = ldf<S>(dec + t * ldd + h);
+      load_run<S, 4, VEC>(v + t * ldv + (size_t)h * dv, col0 + sub * 4, dv, fv);
+      fb = ldf<S>(beta + t * ldb + h);
+    }
+  };
+  fetch(r0);
+
   for (int t0 = r0; t0 < r1; t0 += DS_TB) {
     const int nb = min(DS_TB, r1 - t0);
     __syncthreads();                       // the previous block is consumed
-    // ---- stage: wave w takes tokens w, w+4, ... ----
-    for (int tt = wave; tt < nb; tt += 4) {
-      const size_t t = (size_t)(t0 + tt);
-      const S* qr = q + t * ldq + (size_t)g * dk;
-      const S* kr = k + t * ldk + (size_t)g * dk;
+    // ---- fetched values -> LDS ----
+    if (st < nb) {
       float sq = 0.f, sk = 0.f, qk = 0.f;
-      for (int d = lane; d < dk; d += 64) {
-        const float a = ldf<S>(qr + d), c = ldf<S>(kr + d);
-        sq += a * a;
-        sk += c * c;
-        qk += a * c;
+#pragma unroll
+      for (int j = 0; j < EL; ++j) {
+        sq += fq[j] * fq[j];
+        sk += fk[j] * fk[j];
+        qk += fq[j] * fk[j];
       }
-      sq = wave_sum_f32(sq);
-      sk = wave_sum_f32(sk);
-      qk = wave_sum_f32(qk);
+      sq = row16_sum(sq);
+      sk = row16_sum(sk);
+      qk = row16_sum(qk);
       const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
-      for (int d = lane; d < 4 * RP; d += 64) {
-        const int o = tt * ROW + (d / RP) * RS + (d % RP);
-        const bool in = d < dk;
-        q_s[o] = in ? ldf<S>(qr + d) * rq : 0.f;
-        k_s[o] = in ? ldf<S>(kr + d) * rk : 0.f;
-        if (CH) {
-          float gv = 1.f;
-          if (in) {
-            const float z = ldf<S>(dec + t * ldd + (size_t)h * dk + d) +
-                            dec_bias[(size_t)h * dk + d];
-            gv = expf(-rt * softplus_f32(z));
-          }
-          g_s[o] = gv;
-        }
+      // EL divides RP: a lane's run lies inside one row group's segment
+      const int o = st * ROW + (e0 / RP) * RS + (e0 % RP);
+#pragma unroll
+      for (int j = 0; j < EL; ++j) {
+        q_s[o + j] = fq[j] * rq;
+        k_s[o + j] = fk[j] * rk;
+        if (CH)
+          g_s[o + j] = e0 + j < dk
+              ? exp_s<S>(-rt * softplus_s<S>(fz[j] + bias_r[j])) : 1.f;
       }
-      if (lane == 0) {
-        sc_s[tt * 4 + 0] = 1.0f / (1.0f + expf(-ldf<S>(beta + t * ldb + h)));
-        sc_s[tt * 4 + 1] = qk * rq * rk;
-        if (!CH) {
-          const float z = ldf<S>(dec + t * ldd + h) + dec_bias[h];
-          sc_s[tt * 4 + 2] = expf(-rt * softplus_f32(z));
-        }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v_s[st * 64 + sub * 4 + j] = fv[j];
+      if (sub == 0) {
+        sc_s[st * 4 + 0] = 1.0f / (1.0f + exp_s<S>(-fb));
+        sc_s[st * 4 + 1] = qk * rq * rk;
+        if (!CH) sc_s[st * 4 + 2] = exp_s<S>(-rt * softplus_s<S>(fz[0] + bias_r[0]));
       }
-      const int vc = col0 + lane;
-      v_s[tt * 64 + lane] =
-          vc < dv ? ldf<S>(v + t * ldv + (size_t)h * dv + vc) : 0.f;
     }
     __syncthreads();
+    fetch(t0 + DS_TB);                     // in flight during the walk
     // ---- walk the block: every wave on its own 16 columns ----
     for (int tt = 0; tt < nb; ++tt) {
       const float* kp = k_s + tt * ROW + rg * RS;
@@ -225,6 +279,208 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
       if (row < dk) sp[(size_t)row * dv + col] = s[i];
     }
   }
+}
+
+// Sum over the 16 lanes of a DPP row; every lane gets the total.
+__device__ __forceinline__ float row16_sum_dpp(float v) {
+  // quad_perm [1,0,3,2], [2,3,0,1]: xor 1, xor 2; then rotate the row by 4, 8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));   // row_ror:4
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));   // row_ror:8
+  return v;
+}
+
+// The same recurrence for long chunks (prompts).  Lane = (row group rg =
+// lane & 15, column set lane >> 4): a thread keeps the RP rows rg*RP ..
+// rg*RP+RP-1 (16*RP >= dk) of CPT adjacent columns, so the sums over rows
+// end in four DPP steps inside a 16-lane row and every q / k / decay value
+// read from LDS feeds CPT columns.  A wave covers 4*CPT columns, the
+// workgroup 16*CPT; the host picks CPT so that the launch fills the chip.
+// Staging is the one of delta_scan_kernel: lane `sub` of a token's sixteen
+// stages exactly row group `sub`.
+template <typename S, int RP, bool CH, bool VEC, int CPT>
+__global__ void __launch_bounds__(256) delta_scan_long_kernel(
+    float* __restrict__ out, float* __restrict__ state,
+    const S* __restrict__ q, i64 ldq, const S* __restrict__ k, i64 ldk,
+    const S* __restrict__ v, i64 ldv, const S* __restrict__ beta, i64 ldb,
+    const S* __restrict__ dec, i64 ldd, const float* __restrict__ dec_bias,
+    const float* __restrict__ rate, const i32* __restrict__ cu,
+    const i32* __restrict__ q_start, const i32* __restrict__ sslot, int H,
+    int G, int dk, int dv, float q_scale) {
+  constexpr int ROW = 16 * RP;            // one token's k (or q, or g) in LDS
+  constexpr int NC = 16 * CPT;            // columns of the workgroup
+  __shared__ __attribute__((aligned(16))) float k_s[DS_TB * ROW];
+  __shared__ __attribute__((aligned(16))) float q_s[DS_TB * ROW];
+  __shared__ __attribute__((aligned(16))) float g_s[CH ? DS_TB * ROW : 4];
+  __shared__ __attribute__((aligned(16))) float v_s[DS_TB * NC];
+  __shared__ float sc_s[DS_TB * 4];       // per token: beta, q.k, scalar decay
+
+  const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * NC;
+  const int r0 = cu[b], r1 = cu[b + 1];
+  if (r1 == r0) return;
+  const int g = h / (H / G);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int rg = lane & 15;
+  const int cl = (wave * 4 + (lane >> 4)) * CPT;   // first column in the tile
+  float* sp = state + ((size_t)sslot[b] * H + h) * (size_t)dk * dv;
+
+  float s[CPT][RP];
+#pragma unroll
+  for (int c = 0; c < CPT; ++c)
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+      const int row = rg * RP + i, col = col0 + cl + c;
+      s[c][i] = (q_start[b] > 0 && col < dv && row < dk)
+          ? sp[(size_t)row * dv + col] : 0.f;
+    }
+  const float rt = rate[h];
+
+  // staging role: token st of the block, row group sub
+  const int st = threadIdx.x >> 4, sub = threadIdx.x & 15;
+  const int e0 = sub * RP;
+  float bias_r[CH ? RP : 1];
+  if (CH) {
+#pragma unroll
+    for (int j = 0; j < RP; ++j)
+      bias_r[j] = e0 + j < dk ? dec_bias[(size_t)h * dk + e0 + j] : 0.f;
+  } else {
+    bias_r[0] = dec_bias[h];
+  }
+  float fq[RP], fk[RP], fz[CH ? RP : 1], fv[CPT], fb = 0.f;
+  auto fetch = [&](int t0) {
+    const int tt = t0 + st;
+    if (tt < r1) {
+      const size_t t = (size_t)tt;
+      load_run<S, RP, VEC>(q + t * ldq + (size_t)g * dk, e0, dk, fq);
+      load_run<S, RP, VEC>(k + t * ldk + (size_t)g * dk, e0, dk, fk);
+      if (CH) load_run<S, CH ? RP : 1, VEC>(dec + t * ldd + (size_t)h * dk, e0, dk, fz);
+      else fz[0] = ldf<S>(dec + t * ldd + h);
+      load_run<S, CPT, VEC>(v + t * ldv + (size_t)h * dv, col0 + sub * CPT, dv, fv);
+      fb = ldf<S>(beta + t * ldb + h);
+    }
+  };
+  fetch(r0);
+
+  for (int t0 = r0; t0 < r1; t0 += DS_TB) {
+    const int nb = min(DS_TB, r1 - t0);
+    __syncthreads();                       // the previous block is consumed
+    if (st < nb) {
+      float sq = 0.f, sk = 0.f, qk = 0.f;
+#pragma unroll
+      for (int j = 0; j < RP; ++j) {
+        sq += fq[j] * fq[j];
+        sk += fk[j] * fk[j];
+        qk += fq[j] * fk[j];
+      }
+      sq = row16_sum(sq);
+      sk = row16_sum(sk);
+      qk = row16_sum(qk);
+      const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+      const int o = st * ROW + e0;
+#pragma unroll
+      for (int j = 0; j < RP; ++j) {
+        q_s[o + j] = fq[j] * rq;
+        k_s[o + j] = fk[j] * rk;
+        if (CH)
+          g_s[o + j] = e0 + j < dk
+              ? exp_s<S>(-rt * softplus_s<S>(fz[j] + bias_r[j])) : 1.f;
+      }
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) v_s[st * NC + sub * CPT + j] = fv[j];
+      if (sub == 0) {
+        sc_s[st * 4 + 0] = 1.0f / (1.0f + exp_s<S>(-fb));
+        sc_s[st * 4 + 1] = qk * rq * rk;
+        if (!CH) sc_s[st * 4 + 2] = exp_s<S>(-rt * softplus_s<S>(fz[0] + bias_r[0]));
+      }
+    }
+    __syncthreads();
+    fetch(t0 + DS_TB);                     // in flight during the walk
+    // the next token's LDS values are read while the current one computes
+    float kr[RP], qr[RP], gr[RP], sc[3], vv[CPT];
+    auto read_tok = [&](int tt, float (&kx)[RP], float (&qx)[RP],
+                        float (&gx)[RP], float (&sx)[3], float (&vx)[CPT]) {
+      sx[0] = sc_s[tt * 4 + 0];
+      sx[1] = sc_s[tt * 4 + 1];
+      sx[2] = CH ? 1.f : sc_s[tt * 4 + 2];
+      if constexpr (RP >= 4) {
+#pragma unroll
+        for (int i = 0; i < RP; i += 4) {
+          const f32x4 k4 = *reinterpret_cast<const f32x4*>(k_s + tt * ROW + rg * RP + i);
+          const f32x4 q4 = *reinterpret_cast<const f32x4*>(q_s + tt * ROW + rg * RP + i);
+          f32x4 g4 = f32x4{sx[2], sx[2], sx[2], sx[2]};
+          if (CH) g4 = *reinterpret_cast<const f32x4*>(g_s + tt * ROW + rg * RP + i);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) { kx[i + j] = k4[j]; qx[i + j] = q4[j]; gx[i + j] = g4[j]; }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < RP; ++i) {
+          kx[i] = k_s[tt * ROW + rg * RP + i];
+          qx[i] = q_s[tt * ROW + rg * RP + i];
+          gx[i] = CH ? g_s[tt * ROW + rg * RP + i] : sx[2];
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) vx[c] = v_s[tt * NC + cl + c];
+    };
+    float kn[RP], qn[RP], gn[RP], sn[3], vn[CPT];
+    auto step = [&](int tt, const float (&kx)[RP], const float (&qx)[RP],
+                    const float (&gx)[RP], const float (&sx)[3],
+                    const float (&vx)[CPT], float (&ky)[RP], float (&qy)[RP],
+                    float (&gy)[RP], float (&sy)[3], float (&vy)[CPT]) {
+      read_tok(min(tt + 1, DS_TB - 1), ky, qy, gy, sy, vy);
+      const float bt = sx[0], qk = sx[1];
+      float kd[CPT], qd[CPT];
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        kd[c] = 0.f;
+        qd[c] = 0.f;
+#pragma unroll
+        for (int i = 0; i < RP; ++i) {
+          const float d = s[c][i] * gx[i];
+          s[c][i] = d;
+          kd[c] += kx[i] * d;
+          qd[c] += qx[i] * d;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        kd[c] = row16_sum_dpp(kd[c]);
+        qd[c] = row16_sum_dpp(qd[c]);
+      }
+      float o[CPT];
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        const float u = bt * (vx[c] - kd[c]);
+#pragma unroll
+        for (int i = 0; i < RP; ++i) s[c][i] += kx[i] * u;
+        o[c] = qd[c] + qk * u;
+      }
+      if (rg == 0) {
+        float* op = out + (size_t)(t0 + tt) * ((size_t)H * dv) + (size_t)h * dv + col0 + cl;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c)
+          if (col0 + cl + c < dv) op[c] = o[c];
+      }
+    };
+    read_tok(0, kr, qr, gr, sc, vv);
+    for (int tt = 0; tt < nb; tt += 2) {
+      step(tt, kr, qr, gr, sc, vv, kn, qn, gn, sn, vn);
+      if (tt + 1 < nb) step(tt + 1, kn, qn, gn, sn, vn, kr, qr, gr, sc, vv);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CPT; ++c)
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+      const int row = rg * RP + i, col = col0 + cl + c;
+      if (row < dk && col < dv) sp[(size_t)row * dv + col] = s[c][i];
+    }
 }
 
 // ------------------------------------------------ q/k prep for attention
@@ -390,14 +646,66 @@ AF_EXPORT int afm_delta_scan(
     const void* v, i64 ldv, const void* beta, i64 ldb, const void* dec,
     i64 ldd, const void* dec_bias, const void* rate, const void* cu,
     const void* q_start, const void* sslot, int B, int H, int G, int dk,
-    int dv, int per_channel, float q_scale, int dt, void* stream) {
+    int dv, int per_channel, float q_scale, int long_chunks, int dt,
+    void* stream) {
   if (B == 0) return 0;
   if (H < 1 || G < 1 || H % G != 0 || dk < 1 || dv < 1) return 9003;
   if (dk > 256) return 9004;
   hipStream_t s = (hipStream_t)stream;
+  if (long_chunks) {
+    // prompts: rows over the lanes of a DPP row; as many columns per thread
+    // as still leave two waves per SIMD
+    const bool vecl = dk % 4 == 0 && dv % 4 == 0 && ldq % 4 == 0 &&
+                      ldk % 4 == 0 && ldv % 4 == 0 && ldd % 4 == 0 &&
+                      aligned16(q, k, v, dec);
+    const i64 bh = (i64)B * H;
+    const int cpt = bh * ((dv + 63) / 64) >= 512 ? 4
+                  : bh * ((dv + 31) / 32) >= 512 ? 2 : 1;
+    const dim3 gl(B, H, (dv + 16 * cpt - 1) / (16 * cpt));
+#define DLV(ST, RPV, CHV, VECV, CP)                                         \
+  delta_scan_long_kernel<ST, RPV, CHV, VECV, CP><<<gl, 256, 0, s>>>(        \
+      (float*)out, (float*)state, (const ST*)q, ldq, (const ST*)k, ldk,     \
+      (const ST*)v, ldv, (const ST*)beta, ldb, (const ST*)dec, ldd,         \
+      (const float*)dec_bias, (const float*)rate, (const i32*)cu,           \
+      (const i32*)q_start, (const i32*)sslot, H, G, dk, dv, q_scale)
+#define DL_CP(ST, RPV, CHV, VECV)                                           \
+  do {                                                                      \
+    if (cpt == 4) DLV(ST, RPV, CHV, VECV, 4);                               \
+    else if (cpt == 2) DLV(ST, RPV, CHV, VECV, 2);                          \
+    else DLV(ST, RPV, CHV, VECV, 1);                                        \
+  } while (0)
+#define DL_CH(ST, RPV)                                                      \
+  do {                                                                      \
+    if (per_channel) { if (vecl) DL_CP(ST, RPV, true, true); else DL_CP(ST, RPV, true, false); } \
+    else { if (vecl) DL_CP(ST, RPV, false, true); else DL_CP(ST, RPV, false, false); } \
+  } while (0)
+#define DL_RP(ST)                                    \
+  do {                                               \
+    if (dk <= 16) DL_CH(ST, 1);                      \
+    else if (dk <= 32) DL_CH(ST, 2);                 \
+    else if (dk <= 64) DL_CH(ST, 4);                 \
+    else if (dk <= 128) DL_CH(ST, 8);                \
+    else DL_CH(ST, 16);                              \
+  } while (0)
+    MIX_DISPATCH(dt, DL_RP(u16), DL_RP(float));
+#undef DL_RP
+#undef DL_CH
+#undef DL_CP
+#undef DLV
+    return af_last_err();
+  }
   const dim3 grid(B, H, (dv + 63) / 64);
+  // 4-element vector loads: every head's run of q / k / v / decay logits
+  // starts on an 8- or 16-byte boundary
+  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldq % 4 == 0 &&
+                   ldk % 4 == 0 && ldv % 4 == 0 && ldd % 4 == 0 &&
+                   aligned16(q, k, v, dec);
 #define DSK(ST, RPV, CHV)                                                   \
-  delta_scan_kernel<ST, RPV, CHV><<<grid, 256, 0, s>>>((float*)out,         \
+  do {                                                                      \
+    if (vec) DSKV(ST, RPV, CHV, true); else DSKV(ST, RPV, CHV, false);      \
+  } while (0)
+#define DSKV(ST, RPV, CHV, VECV)                                            \
+  delta_scan_kernel<ST, RPV, CHV, VECV><<<grid, 256, 0, s>>>((float*)out,   \
       (float*)state, (const ST*)q, ldq, (const ST*)k, ldk, (const ST*)v,    \
       ldv, (const ST*)beta, ldb, (const ST*)dec, ldd,                       \
       (const float*)dec_bias, (const float*)rate, (const i32*)cu,           \
@@ -419,6 +727,7 @@ AF_EXPORT int afm_delta_scan(
 #undef DSK_RP
 #undef DSK_CH
 #undef DSK
+#undef DSKV
   return af_last_err();
 }
 

@@ -188,7 +188,7 @@ def _mix_sigs() -> dict:
         },
         "delta": {
             "afm_delta_scan": [p, p, p, i64, p, i64, p, i64, p, i64, p, i64,
-                               p, p, p, p, p, i, i, i, i, i, i, f, i, p],
+                               p, p, p, p, p, i, i, i, i, i, i, f, i, i, p],
             "afm_qk_rope_cache": [p, p, i64, p, i64, p, i64, p, p, p, p, p,
                                   p, i, p, p, p, p, f, i, i, i, i, i, i, i,
                                   p],

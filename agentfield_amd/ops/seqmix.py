@@ -1269,6 +1269,11 @@ def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     return out
 
 
+# a step whose longest row chunk reaches this many rows runs the delta rule
+# in its prompt layout (rows of the state over the lanes of a DPP row)
+DELTA_LONG_ROWS = 32
+
+
 def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                beta: torch.Tensor, decay: torch.Tensor,
                decay_bias: torch.Tensor, rate: torch.Tensor,
@@ -1328,13 +1333,19 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         return out.view(T, H * dv)
     out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
     B = md.q_start.numel()
+    # prompt portions amortise the state's load and store over many tokens
+    # and take the layout with the shortest per-token chain; short chunks and
+    # decode steps take the one whose state accesses coalesce
+    lens = getattr(md, "seq_lens", None)
+    long_chunks = lens is not None and max(lens) >= DELTA_LONG_ROWS
     rc = _L().afm_delta_scan(
         _lib.ptr(out), _lib.ptr(state), _lib.ptr(q), _rowstride(q),
         _lib.ptr(k), _rowstride(k), _lib.ptr(v), _rowstride(v),
         _lib.ptr(beta), _rowstride(beta), _lib.ptr(decay), _rowstride(decay),
         _lib.ptr(decay_bias), _lib.ptr(rate), _lib.ptr(md.cu_seqlens),
         _lib.ptr(md.q_start), _lib.ptr(md.state_slots), B, H, G, dk, dv,
-        1 if per_channel else 0, float(q_scale), _code(q), _lib.cur_stream())
+        1 if per_channel else 0, float(q_scale), 1 if long_chunks else 0,
+        _code(q), _lib.cur_stream())
     _lib.check(rc, "afm_delta_scan")
     return out
 

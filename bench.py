@@ -80,7 +80,7 @@ def parse_args():
     p.add_argument("--family-compare", action="store_true",
                    help="instead of the default workload: engine-level "
                         "prefill and decode token throughput of the hybrid "
-                        "families (Reperax, Zudisun, Fugevik) beside each other and "
+                        "families (Reperax, Zudisun, Fugevik, Vabedra) beside each other and "
                         "the Llama family at equal width / ff / depth, "
                         "random weights; one JSON line per model and phase "
                         "(single GPU)")

@@ -268,7 +268,8 @@ def test_delta_scan_alone(device, dtype, per_channel, shape):
             q.repeat_interleave(H // G, 1), k.repeat_interleave(H // G, 1),
             s["v"].to(F64).view(T, H, dv), torch.sigmoid(s["b"].to(F64)),
             g).reshape(T, H * dv))
-    cuts = [(0, 0), (5, 2), (7, 3), (30, 19), (31, 37), (61, 37)]
+    # one step long enough for the prompt layout, the others short
+    cuts = [(0, 0), (5, 2), (7, 3), (45, 19), (46, 37), (61, 37)]
     got = [[], []]
     for (a0, b0), (a1, b1) in zip(cuts[:-1], cuts[1:]):
         parts = [(i, lo, hi) for i, (lo, hi) in enumerate(((a0, a1),
