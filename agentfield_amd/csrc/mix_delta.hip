@@ -484,37 +484,68 @@ __global__ void __launch_bounds__(256) delta_scan_long_kernel(
 }
 
 // ------------------------------------------------ q/k prep for attention
-// One workgroup per row.  Every q head and k head: + bias, RMSNorm over the
-// head with a weight shared by heads, rotate-half rotary positions on the
-// first `rot` dims (dim i pairs with i + rot/2; angle = position * f_i, the
-// product and its sine / cosine taken in double precision).  q goes to a
-// contiguous [T, H*dk] buffer, k and v (+ bias) to their pages.
-template <typename S>
+// cos | sin of position * f_i per row, the product and the functions taken
+// in double precision: tab [T, 2*half] fp32.  One table serves every layer
+// of a step that rotates with the same frequencies.
+__global__ void __launch_bounds__(256) rotary_table_kernel(
+    float* __restrict__ tab, const i32* __restrict__ positions,
+    const double* __restrict__ inv_freq, i64 n, int half) {
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    const i64 t = i / half;
+    const int j = (int)(i % half);
+    const double a = (double)positions[t] * inv_freq[j];
+    tab[t * 2 * half + j] = (float)cos(a);
+    tab[t * 2 * half + half + j] = (float)sin(a);
+  }
+}
+
+// 2 consecutive elements (V2) or one
+template <typename S, bool V2>
+__device__ __forceinline__ void ld2(const S* p, float& a, float& b) {
+  if constexpr (!V2) { a = ldf<S>(p); b = 0.f; }
+  else if constexpr (sizeof(S) == 2) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    a = bf2f((u16)(w & 0xffffu));
+    b = bf2f((u16)(w >> 16));
+  } else {
+    const f32x2 w = *reinterpret_cast<const f32x2*>(p);
+    a = w[0];
+    b = w[1];
+  }
+}
+template <typename S, bool V2>
+__device__ __forceinline__ void st2(S* p, float a, float b) {
+  if constexpr (!V2) stf<S>(p, a);
+  else if constexpr (sizeof(S) == 2)
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)f2bf(a) | ((uint32_t)f2bf(b) << 16);
+  else *reinterpret_cast<f32x2*>(p) = f32x2{a, b};
+}
+
+// One workgroup per row, one wave per head at a time.  Every q head and k
+// head: + bias, RMSNorm over the head with a weight shared by heads,
+// rotate-half rotary positions on the first `rot` dims (dim i pairs with
+// i + rot/2) with the row's cos | sin from `tab`.  q goes to a contiguous
+// [T, H*dk] buffer, k and v (+ bias) to their pages.  V2: two adjacent
+// elements per lane and access (even sizes, 4- / 8-byte aligned rows).
+template <typename S, bool V2>
 __global__ void __launch_bounds__(256) qk_rope_cache_kernel(
     S* __restrict__ qo, const S* __restrict__ q, i64 ldq,
     const S* __restrict__ k, i64 ldk, const S* __restrict__ v, i64 ldv,
     const S* __restrict__ qb, const S* __restrict__ kb,
     const S* __restrict__ vb, const S* __restrict__ qw,
-    const S* __restrict__ kw, const double* __restrict__ inv_freq, int rot,
-    const i32* __restrict__ positions, S* __restrict__ kc, S* __restrict__ vc,
-    const i64* __restrict__ slots, float eps, int H, int G, int dk, int dv,
-    int page) {
-  extern __shared__ float sm[];
+    const S* __restrict__ kw, const float* __restrict__ tab, int rot,
+    S* __restrict__ kc, S* __restrict__ vc, const i64* __restrict__ slots,
+    float eps, int H, int G, int dk, int dv, int page) {
+  extern __shared__ float sm[];            // [4][dk]
+  constexpr int E = V2 ? 2 : 1;
   const int half = rot / 2;
-  float* cs = sm;                          // [half] cos, [half] sin
-  float* buf = sm + 2 * half;              // [4][dk]
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pos = positions[t];
-  for (int i = threadIdx.x; i < half; i += 256) {
-    const double a = (double)pos * inv_freq[i];
-    cs[i] = (float)cos(a);
-    cs[half + i] = (float)sin(a);
-  }
-  __syncthreads();
+  const float* cs = tab + (size_t)t * rot;  // [half] cos, [half] sin
   const i64 sl = slots[t];
   const i64 pg = sl / page, off = sl % page;
-  float* nb = buf + wave * dk;
+  float* nb = sm + wave * dk;
   for (int u = wave; u < H + G; u += 4) {
     const bool isq = u < H;
     const int hh = isq ? u : u - H;
@@ -523,33 +554,50 @@ __global__ void __launch_bounds__(256) qk_rope_cache_kernel(
     const S* bias = isq ? qb : kb;
     const S* w = isq ? qw : kw;
     float ss = 0.f;
-    for (int d = lane; d < dk; d += 64) {
-      float x = ldf<S>(src + d);
-      if (bias) x += ldf<S>(bias + (size_t)hh * dk + d);
-      nb[d] = x;
-      ss += x * x;
+    for (int d = lane * E; d < dk; d += 64 * E) {
+      float x0, x1, b0 = 0.f, b1 = 0.f;
+      ld2<S, V2>(src + d, x0, x1);
+      if (bias) ld2<S, V2>(bias + (size_t)hh * dk + d, b0, b1);
+      x0 += b0;
+      x1 += b1;
+      nb[d] = x0;
+      if (V2) nb[d + 1] = x1;
+      ss += x0 * x0 + x1 * x1;
     }
     ss = wave_sum_f32(ss);
     const float r = w ? 1.0f / sqrtf(ss / (float)dk + eps) : 1.0f;
-    __builtin_amdgcn_wave_barrier();
-    for (int d = lane; d < dk; d += 64)
-      nb[d] = nb[d] * r * (w ? ldf<S>(w + d) : 1.0f);
-    __builtin_amdgcn_wave_barrier();
+    for (int d = lane * E; d < dk; d += 64 * E) {
+      float w0 = 1.f, w1 = 1.f;
+      if (w) ld2<S, V2>(w + d, w0, w1);
+      nb[d] = nb[d] * r * w0;              // each lane rewrites its own slots
+      if (V2) nb[d + 1] = nb[d + 1] * r * w1;
+    }
+    __builtin_amdgcn_wave_barrier();       // partners come from other lanes
     S* dst = isq ? qo + ((size_t)t * H + hh) * dk
                  : kc + (((size_t)pg * G + hh) * page + off) * dk;
-    for (int d = lane; d < dk; d += 64) {
-      float o = nb[d];
-      if (d < half) o = o * cs[d] - nb[d + half] * cs[half + d];
-      else if (d < rot) o = o * cs[d - half] + nb[d - half] * cs[d];
-      if (isq || sl >= 0) stf<S>(dst + d, o);
+    if (isq || sl >= 0) {
+      for (int d = lane * E; d < dk; d += 64 * E) {
+        float o[2];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int dd = d + e;
+          float x = nb[dd];
+          if (dd < half) x = x * cs[dd] - nb[dd + half] * cs[half + dd];
+          else if (dd < rot) x = x * cs[dd - half] + nb[dd - half] * cs[dd];
+          o[e] = x;
+        }
+        st2<S, V2>(dst + d, o[0], V2 ? o[1] : 0.f);
+      }
     }
-    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_wave_barrier();       // the buffer is reused
   }
   if (sl < 0) return;
-  for (int i = threadIdx.x; i < G * dv; i += 256) {
-    float x = ldf<S>(v + (size_t)t * ldv + i);
-    if (vb) x += ldf<S>(vb + i);
-    stf<S>(vc + (((size_t)pg * G + i / dv) * page + off) * dv + (i % dv), x);
+  for (int i = threadIdx.x * E; i < G * dv; i += 256 * E) {
+    float x0, x1, b0 = 0.f, b1 = 0.f;
+    ld2<S, V2>(v + (size_t)t * ldv + i, x0, x1);
+    if (vb) ld2<S, V2>(vb + i, b0, b1);
+    st2<S, V2>(vc + (((size_t)pg * G + i / dv) * page + off) * dv + (i % dv),
+               x0 + b0, x1 + b1);
   }
 }
 
@@ -557,7 +605,11 @@ __global__ void __launch_bounds__(256) qk_rope_cache_kernel(
 // x <- (alpha x + u) / rms(alpha x + u) * w in place on the fp32 residual,
 // also written as h in the storage dtype.  u = y, or with a second branch
 // u = (y / rms(y) * wy + y2 / rms(y2) * wy2) / 2.
-template <typename S, typename YT, int V>
+// REG: the row fits 8 passes of the workgroup and waits in registers
+// between the sum and the norm; otherwise it waits in x itself.
+constexpr int PNS_IT = 8;
+
+template <typename S, typename YT, int V, bool REG>
 __global__ void __launch_bounds__(256) postnorm_sum_kernel(
     float* __restrict__ x, S* __restrict__ h, const YT* __restrict__ y,
     i64 ldy, const YT* __restrict__ y2, i64 ldy2, const S* __restrict__ wy,
@@ -583,8 +635,9 @@ __global__ void __launch_bounds__(256) postnorm_sum_kernel(
     r2 = 0.5f / sqrtf(ss[1] / (float)W + eps);
   }
   float sv[1] = {0.f};
-  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
-    float a[4], xv[4];
+  float keep[REG ? PNS_IT : 1][4];
+  auto sum_at = [&](int i, float (&xv)[4]) {
+    float a[4];
     ldv<YT, V>(yr + i, a);
     ldv<float, V>(xr + i, xv);
     if (y2r) {
@@ -600,18 +653,42 @@ __global__ void __launch_bounds__(256) postnorm_sum_kernel(
       xv[j] = alpha * xv[j] + a[j];
       sv[0] += xv[j] * xv[j];
     }
-    stv<float, V>(xr + i, xv);          // re-read below by the same thread
+  };
+  if constexpr (REG) {
+#pragma unroll
+    for (int it = 0; it < PNS_IT; ++it) {
+      const int i = (it * 256 + threadIdx.x) * V;
+      if (i < W) sum_at(i, keep[it]);
+    }
+  } else {
+    for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+      float xv[4];
+      sum_at(i, xv);
+      stv<float, V>(xr + i, xv);          // re-read below by the same thread
+    }
   }
   block_sum<1>(sv, red);
   const float r = 1.0f / sqrtf(sv[0] / (float)W + eps);
-  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
-    float xv[4], wv[4];
-    ldv<float, V>(xr + i, xv);
+  auto norm_at = [&](int i, float (&xv)[4]) {
+    float wv[4];
     ldv<S, V>(w + i, wv);
 #pragma unroll
     for (int j = 0; j < V; ++j) xv[j] = xv[j] * r * wv[j];
     stv<float, V>(xr + i, xv);
     if (h) stv<S, V>(h + (size_t)t * W + i, xv);
+  };
+  if constexpr (REG) {
+#pragma unroll
+    for (int it = 0; it < PNS_IT; ++it) {
+      const int i = (it * 256 + threadIdx.x) * V;
+      if (i < W) norm_at(i, keep[it]);
+    }
+  } else {
+    for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+      float xv[4];
+      ldv<float, V>(xr + i, xv);
+      norm_at(i, xv);
+    }
   }
 }
 
@@ -731,24 +808,40 @@ AF_EXPORT int afm_delta_scan(
   return af_last_err();
 }
 
+AF_EXPORT int afm_rotary_table(void* tab, const void* positions,
+                               const void* inv_freq, int T, int half,
+                               void* stream) {
+  if (T == 0 || half == 0) return 0;
+  const i64 n = (i64)T * half;
+  rotary_table_kernel<<<grid_for(n), 256, 0, (hipStream_t)stream>>>(
+      (float*)tab, (const i32*)positions, (const double*)inv_freq, n, half);
+  return af_last_err();
+}
+
 AF_EXPORT int afm_qk_rope_cache(
     void* qo, const void* q, i64 ldq, const void* k, i64 ldk, const void* v,
     i64 ldv, const void* qb, const void* kb, const void* vb, const void* qw,
-    const void* kw, const void* inv_freq, int rot, const void* positions,
-    void* kc, void* vc, const void* slots, float eps, int T, int H, int G,
-    int dk, int dv, int page, int dt, void* stream) {
+    const void* kw, const void* tab, int rot, void* kc, void* vc,
+    const void* slots, float eps, int T, int H, int G, int dk, int dv,
+    int page, int dt, void* stream) {
   if (T == 0) return 0;
-  if (rot < 0 || rot > dk || rot % 2 != 0) return 9003;
-  const size_t smem = (size_t)(rot + 4 * dk) * sizeof(float);
+  if (rot < 0 || rot > dk || rot % 2 != 0 || (rot > 0 && !tab)) return 9003;
+  const size_t smem = (size_t)(4 * dk) * sizeof(float);
   if (smem > 60000) return 9004;
   hipStream_t s = (hipStream_t)stream;
-#define QRC(ST)                                                              \
-  qk_rope_cache_kernel<ST><<<T, 256, smem, s>>>((ST*)qo, (const ST*)q, ldq,  \
-      (const ST*)k, ldk, (const ST*)v, ldv, (const ST*)qb, (const ST*)kb,    \
-      (const ST*)vb, (const ST*)qw, (const ST*)kw, (const double*)inv_freq,  \
-      rot, (const i32*)positions, (ST*)kc, (ST*)vc, (const i64*)slots, eps,  \
-      H, G, dk, dv, page)
-  MIX_DISPATCH(dt, (QRC(u16)), (QRC(float)));
+  const size_t al = dt == 0 ? 4 : 8;       // bytes of an element pair
+  auto ok = [&](const void* p) { return (uintptr_t)p % al == 0; };
+  const bool v2 = dk % 2 == 0 && dv % 2 == 0 && ldq % 2 == 0 && ldk % 2 == 0 &&
+                  ldv % 2 == 0 && ok(qo) && ok(q) && ok(k) && ok(v) && ok(qb) &&
+                  ok(kb) && ok(vb) && ok(qw) && ok(kw) && ok(kc) && ok(vc);
+#define QRC(ST, V2)                                                          \
+  qk_rope_cache_kernel<ST, V2><<<T, 256, smem, s>>>((ST*)qo, (const ST*)q,   \
+      ldq, (const ST*)k, ldk, (const ST*)v, ldv, (const ST*)qb,              \
+      (const ST*)kb, (const ST*)vb, (const ST*)qw, (const ST*)kw,            \
+      (const float*)tab, rot, (ST*)kc, (ST*)vc, (const i64*)slots, eps, H,   \
+      G, dk, dv, page)
+  if (v2) MIX_DISPATCH(dt, (QRC(u16, true)), (QRC(float, true)));
+  else MIX_DISPATCH(dt, (QRC(u16, false)), (QRC(float, false)));
 #undef QRC
   return af_last_err();
 }
@@ -763,16 +856,15 @@ AF_EXPORT int afm_postnorm_sum(void* x, void* h, const void* y, i64 ldy,
   hipStream_t s = (hipStream_t)stream;
   const bool vec = W % 4 == 0 && ldy % 4 == 0 && ldy2 % 4 == 0 &&
                    aligned16(x, h, y, y2, wy, wy2, w);
+  const bool reg = W <= PNS_IT * 256 * (vec ? 4 : 1);
+#define PNSK(ST, YT, V, R)                                                   \
+  postnorm_sum_kernel<ST, YT, V, R><<<T, 256, 0, s>>>((float*)x, (ST*)h,     \
+      (const YT*)y, ldy, (const YT*)y2, ldy2, (const ST*)wy, (const ST*)wy2, \
+      (const ST*)w, alpha, eps, W)
 #define PNS(ST, YT)                                                          \
   do {                                                                       \
-    if (vec)                                                                 \
-      postnorm_sum_kernel<ST, YT, 4><<<T, 256, 0, s>>>((float*)x, (ST*)h,    \
-          (const YT*)y, ldy, (const YT*)y2, ldy2, (const ST*)wy,             \
-          (const ST*)wy2, (const ST*)w, alpha, eps, W);                      \
-    else                                                                     \
-      postnorm_sum_kernel<ST, YT, 1><<<T, 256, 0, s>>>((float*)x, (ST*)h,    \
-          (const YT*)y, ldy, (const YT*)y2, ldy2, (const ST*)wy,             \
-          (const ST*)wy2, (const ST*)w, alpha, eps, W);                      \
+    if (vec) { if (reg) PNSK(ST, YT, 4, true); else PNSK(ST, YT, 4, false); } \
+    else { if (reg) PNSK(ST, YT, 1, true); else PNSK(ST, YT, 1, false); }    \
   } while (0)
   if (dt == 0) {
     if (y_f32) PNS(u16, float);
@@ -783,6 +875,7 @@ AF_EXPORT int afm_postnorm_sum(void* x, void* h, const void* y, i64 ldy,
     return 9002;
   }
 #undef PNS
+#undef PNSK
   return af_last_err();
 }
 

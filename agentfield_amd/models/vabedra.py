@@ -323,15 +323,23 @@ class SinkWindowAttention(nn.Module):
     def in_rows(self) -> int:
         return self.nq + self.nk + self.nv
 
-    def forward(self, p, cache: HybridCache, run: int, md, positions):
+    def forward(self, p, cache: HybridCache, run: int, md, positions, ctx):
         s = self.spec
         a, b, c = self.nq, self.nq + self.nk, self.nq + self.nk + self.nv
+        tab = None
+        if self.inv_freq is not None:
+            # layers that rotate alike share the step's cos / sin table
+            key = (s.rot_dims, s.rot_base,
+                   tuple(sorted((s.rot_scaling or {}).items())))
+            tab = ctx.get(key)
+            if tab is None:
+                tab = ctx[key] = sm.rotary_table(positions, self.inv_freq)
         q = sm.qk_rope_cache(
             p[:, :a], p[:, a:b], p[:, b:c], s.heads, s.kv_heads, self.eps,
             cache.k[run], cache.v[run], md.slots, positions,
             q_bias=self.bias[:a], k_bias=self.bias[a:b],
             v_bias=self.bias[b:c], q_norm=self.q_norm, k_norm=self.k_norm,
-            inv_freq=self.inv_freq)
+            rot_tab=tab)
         o = sm.masked_attention(q, cache.k[run], cache.v[run], md, positions,
                                 s.scale, s.heads, window=s.window,
                                 sink=self.sink, softcap=s.softcap,
@@ -369,14 +377,14 @@ class VabedraLayer(nn.Module):
             self.side_proj = nn.Parameter(torch.empty(W, cfg.side_dim))
             self.side_norm = nn.Parameter(torch.empty(W))
 
-    def forward(self, x, h, ids, side_table, cache, run, md, positions):
+    def forward(self, x, h, ids, side_table, cache, run, md, positions, ctx):
         """x: fp32 residual (updated in place); h: x in the model dtype.
         Returns the new h."""
         dt = self.norm1.dtype
         p = sm.matmul(h, self.mix_in)
         if self.attn is not None:
             n = self.attn.in_rows()
-            left = self.attn(p[:, :n], cache, run, md, positions)
+            left = self.attn(p[:, :n], cache, run, md, positions, ctx)
             right = self.delta(p[:, n:], cache, run, md)
             h = sm.postnorm_sum(x, left, self.alpha, self.norm1, self.eps, dt,
                                 y2=right, wy=self.left_out,
@@ -442,8 +450,10 @@ class VabedraForCausalLM(nn.Module):
         dt = self.embed.dtype
         x = sm.embed_rows(ids, self.embed, scale=self.cfg.embed_scale)
         h = sm.cast_rows(x, dt)
+        ctx: dict = {}
         for run, layer in enumerate(self.layers):
-            h = layer(x, h, ids, self.side_embed, cache, run, md, positions)
+            h = layer(x, h, ids, self.side_embed, cache, run, md, positions,
+                      ctx)
             if self.record_runs is not None:
                 self.record_runs.append(x.clone())
         hn = sm.norm_rows(x, self.final_norm, self.cfg.eps, logit_rows, dt,

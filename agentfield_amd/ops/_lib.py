@@ -189,9 +189,9 @@ def _mix_sigs() -> dict:
         "delta": {
             "afm_delta_scan": [p, p, p, i64, p, i64, p, i64, p, i64, p, i64,
                                p, p, p, p, p, i, i, i, i, i, i, f, i, i, p],
+            "afm_rotary_table": [p, p, p, i, i, p],
             "afm_qk_rope_cache": [p, p, i64, p, i64, p, i64, p, p, p, p, p,
-                                  p, i, p, p, p, p, f, i, i, i, i, i, i, i,
-                                  p],
+                                  p, i, p, p, p, f, i, i, i, i, i, i, i, p],
             "afm_postnorm_sum": [p, p, p, i64, i, p, i64, p, p, p, f, f, i,
                                  i, i, p],
             "afm_gate_gather": [p, p, i64, p, i64, i, p, i, i, i, p],

@@ -1202,6 +1202,24 @@ def scaled_inv_freq(dims: int, base: float,
     return torch.tensor(out, dtype=torch.float64)
 
 
+def rotary_table(positions: torch.Tensor,
+                 inv_freq: torch.Tensor) -> torch.Tensor:
+    """[cos | sin] of position * f_i per row as fp32 [T, 2*len(inv_freq)];
+    inv_freq float64, the product and the functions in double precision.
+    One table serves every layer of a step that rotates alike."""
+    T, half = positions.numel(), inv_freq.numel()
+    if not _gpu(positions):
+        ang = positions.double()[:, None] * inv_freq.double()[None]
+        return torch.cat([ang.cos(), ang.sin()], 1).float()
+    tab = torch.empty(T, 2 * half, dtype=torch.float32,
+                      device=positions.device)
+    rc = _L().afm_rotary_table(_lib.ptr(tab), _lib.ptr(positions),
+                               _lib.ptr(inv_freq), T, half,
+                               _lib.cur_stream())
+    _lib.check(rc, "afm_rotary_table")
+    return tab
+
+
 def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                   heads: int, kv_heads: int, eps: float,
                   kcache: torch.Tensor, vcache: torch.Tensor,
@@ -1211,21 +1229,24 @@ def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                   v_bias: torch.Tensor | None = None,
                   q_norm: torch.Tensor | None = None,
                   k_norm: torch.Tensor | None = None,
-                  inv_freq: torch.Tensor | None = None) -> torch.Tensor:
+                  inv_freq: torch.Tensor | None = None,
+                  rot_tab: torch.Tensor | None = None) -> torch.Tensor:
     """Row steps in front of rotary attention.  q [T, H*dk], k [T, G*dk], v
     [T, G*dv] (strided views allowed) get their biases; every q and k head
     is RMS-normed over dk with a plain weight [dk] shared by heads (skipped
     without one); the first 2*len(inv_freq) dims of each head are rotated,
     dim i paired with i + len(inv_freq), by the angle position * f_i
-    (inv_freq float64; product, sine and cosine in double precision); k and
-    v are appended to the paged caches at `slots`.  Returns q, contiguous
-    [T, H*dk]."""
+    (inv_freq float64; product, sine and cosine in double precision; or the
+    rows' ready rotary_table as rot_tab); k and v are appended to the paged
+    caches at `slots`.  Returns q, contiguous [T, H*dk]."""
     T = q.shape[0]
     H, G = heads, kv_heads
     dk = q.shape[1] // H
     dv = v.shape[1] // G
     page = kcache.shape[2]
-    half = inv_freq.numel() if inv_freq is not None else 0
+    if rot_tab is None and inv_freq is not None and inv_freq.numel() > 0:
+        rot_tab = rotary_table(positions, inv_freq)
+    half = rot_tab.shape[1] // 2 if rot_tab is not None else 0
     if not _gpu(q):
         qf = q.float()
         kf = k.float()
@@ -1244,8 +1265,7 @@ def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) \
                 * k_norm.float()
         if half:
-            ang = positions.double()[:, None] * inv_freq.double()[None]
-            c, s = ang.cos().float()[:, None], ang.sin().float()[:, None]
+            c, s = rot_tab[:, None, :half], rot_tab[:, None, half:]
 
             def rot(x):
                 u, w = x[..., :half], x[..., half:2 * half]
@@ -1262,9 +1282,9 @@ def qk_rope_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         _lib.ptr(out), _lib.ptr(q), _rowstride(q), _lib.ptr(k), _rowstride(k),
         _lib.ptr(v), _rowstride(v), _lib.ptr(q_bias), _lib.ptr(k_bias),
         _lib.ptr(v_bias), _lib.ptr(q_norm), _lib.ptr(k_norm),
-        _lib.ptr(inv_freq), 2 * half, _lib.ptr(positions), _lib.ptr(kcache),
-        _lib.ptr(vcache), _lib.ptr(slots), float(eps), T, H, G, dk, dv, page,
-        _code(q), _lib.cur_stream())
+        _lib.ptr(rot_tab), 2 * half, _lib.ptr(kcache), _lib.ptr(vcache),
+        _lib.ptr(slots), float(eps), T, H, G, dk, dv, page, _code(q),
+        _lib.cur_stream())
     _lib.check(rc, "afm_qk_rope_cache")
     return out
 

@@ -542,7 +542,7 @@ def test_bounded_experts_both_dispatches(device, dtype, T):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W", [32, 30, 1028])
+@pytest.mark.parametrize("W", [32, 30, 1028, 2050, 8196])
 def test_postnorm_sum_and_side_input(device, dtype, W):
     torch.manual_seed(W)
     T, eps, alpha, V, sd = 9, 1e-5, 1.7, 11, 3
