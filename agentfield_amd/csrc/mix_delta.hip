@@ -601,6 +601,112 @@ __global__ void __launch_bounds__(256) qk_rope_cache_kernel(
   }
 }
 
+// The same for even head sizes up to 128 * NP with aligned rows: a lane owns
+// NP element pairs of every head, so its norm weights, cos / sin factors and
+// rotation partners are fixed for the row and sit in registers; the next
+// head's values are loaded while the current head is reduced and rotated.
+template <typename S, int NP>
+__global__ void __launch_bounds__(256) qk_rope_cache_pairs_kernel(
+    S* __restrict__ qo, const S* __restrict__ q, i64 ldq,
+    const S* __restrict__ k, i64 ldk, const S* __restrict__ v, i64 ldv,
+    const S* __restrict__ qb, const S* __restrict__ kb,
+    const S* __restrict__ vb, const S* __restrict__ qw,
+    const S* __restrict__ kw, const float* __restrict__ tab, int rot,
+    S* __restrict__ kc, S* __restrict__ vc, const i64* __restrict__ slots,
+    float eps, int H, int G, int dk, int dv, int page) {
+  extern __shared__ float sm[];            // [4][dk]
+  const int half = rot / 2;
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float* cs = tab + (size_t)t * rot;
+  const i64 sl = slots[t];
+  const i64 pg = sl / page, off = sl % page;
+  float* nb = sm + wave * dk;
+  // per-lane constants of the row: o = n[d] * cc + n[pi] * sn
+  float cc[NP][2], sn[NP][2], wq[NP][2], wk[NP][2];
+  int pi[NP][2];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int d = lane * 2 + 128 * p;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int dd = d + e;
+      cc[p][e] = 1.f; sn[p][e] = 0.f; pi[p][e] = dd < dk ? dd : 0;
+      if (dd < half) { cc[p][e] = cs[dd]; sn[p][e] = -cs[half + dd]; pi[p][e] = dd + half; }
+      else if (dd < rot) { cc[p][e] = cs[dd - half]; sn[p][e] = cs[dd]; pi[p][e] = dd - half; }
+    }
+    wq[p][0] = wq[p][1] = wk[p][0] = wk[p][1] = 1.f;
+    if (d < dk) {
+      if (qw) ld2<S, true>(qw + d, wq[p][0], wq[p][1]);
+      if (kw) ld2<S, true>(kw + d, wk[p][0], wk[p][1]);
+    }
+  }
+  auto fetch = [&](int u, float (&x)[NP][2]) {
+    const bool isq = u < H;
+    const int hh = isq ? u : u - H;
+    const S* src = isq ? q + (size_t)t * ldq + (size_t)hh * dk
+                       : k + (size_t)t * ldk + (size_t)hh * dk;
+    const S* bias = isq ? qb : kb;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int d = lane * 2 + 128 * p;
+      x[p][0] = x[p][1] = 0.f;
+      if (d < dk) {
+        ld2<S, true>(src + d, x[p][0], x[p][1]);
+        if (bias) {
+          float b0, b1;
+          ld2<S, true>(bias + (size_t)hh * dk + d, b0, b1);
+          x[p][0] += b0;
+          x[p][1] += b1;
+        }
+      }
+    }
+  };
+  float cur[NP][2], nxt[NP][2];
+  if (wave < H + G) fetch(wave, cur);
+  for (int u = wave; u < H + G; u += 4) {
+    if (u + 4 < H + G) fetch(u + 4, nxt);
+    const bool isq = u < H;
+    const int hh = isq ? u : u - H;
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) ss += cur[p][0] * cur[p][0] + cur[p][1] * cur[p][1];
+    ss = wave_sum_f32(ss);
+    const float r = (isq ? qw : kw) ? 1.0f / sqrtf(ss / (float)dk + eps) : 1.0f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int d = lane * 2 + 128 * p;
+      if (d < dk) {
+        nb[d] = cur[p][0] * r * (isq ? wq[p][0] : wk[p][0]);
+        nb[d + 1] = cur[p][1] * r * (isq ? wq[p][1] : wk[p][1]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();       // partners come from other lanes
+    S* dst = isq ? qo + ((size_t)t * H + hh) * dk
+                 : kc + (((size_t)pg * G + hh) * page + off) * dk;
+    if (isq || sl >= 0) {
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        const int d = lane * 2 + 128 * p;
+        if (d < dk)
+          st2<S, true>(dst + d, nb[d] * cc[p][0] + nb[pi[p][0]] * sn[p][0],
+                       nb[d + 1] * cc[p][1] + nb[pi[p][1]] * sn[p][1]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();       // the buffer is reused
+#pragma unroll
+    for (int p = 0; p < NP; ++p) { cur[p][0] = nxt[p][0]; cur[p][1] = nxt[p][1]; }
+  }
+  if (sl < 0) return;
+  for (int i = threadIdx.x * 2; i < G * dv; i += 512) {
+    float x0, x1, b0 = 0.f, b1 = 0.f;
+    ld2<S, true>(v + (size_t)t * ldv + i, x0, x1);
+    if (vb) ld2<S, true>(vb + i, b0, b1);
+    st2<S, true>(vc + (((size_t)pg * G + i / dv) * page + off) * dv + (i % dv),
+                 x0 + b0, x1 + b1);
+  }
+}
+
 // --------------------------------------------------------- postnorm sum
 // x <- (alpha x + u) / rms(alpha x + u) * w in place on the fp32 residual,
 // also written as h in the storage dtype.  u = y, or with a second branch
@@ -840,8 +946,17 @@ AF_EXPORT int afm_qk_rope_cache(
       (const ST*)kb, (const ST*)vb, (const ST*)qw, (const ST*)kw,            \
       (const float*)tab, rot, (ST*)kc, (ST*)vc, (const i64*)slots, eps, H,   \
       G, dk, dv, page)
-  if (v2) MIX_DISPATCH(dt, (QRC(u16, true)), (QRC(float, true)));
+#define QRP(ST, NPV)                                                         \
+  qk_rope_cache_pairs_kernel<ST, NPV><<<T, 256, smem, s>>>((ST*)qo,          \
+      (const ST*)q, ldq, (const ST*)k, ldk, (const ST*)v, ldv,               \
+      (const ST*)qb, (const ST*)kb, (const ST*)vb, (const ST*)qw,            \
+      (const ST*)kw, (const float*)tab, rot, (ST*)kc, (ST*)vc,               \
+      (const i64*)slots, eps, H, G, dk, dv, page)
+  if (v2 && dk <= 128) MIX_DISPATCH(dt, (QRP(u16, 1)), (QRP(float, 1)));
+  else if (v2 && dk <= 256) MIX_DISPATCH(dt, (QRP(u16, 2)), (QRP(float, 2)));
+  else if (v2) MIX_DISPATCH(dt, (QRC(u16, true)), (QRC(float, true)));
   else MIX_DISPATCH(dt, (QRC(u16, false)), (QRC(float, false)));
+#undef QRP
 #undef QRC
   return af_last_err();
 }

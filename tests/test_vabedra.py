@@ -366,7 +366,7 @@ def test_scaled_frequencies_three_regimes():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [(4, 2, 16, 8, 6), (1, 1, 8, 8, 8),
                                   (9, 3, 6, 10, 2), (2, 2, 70, 24, 0),
-                                  (3, 1, 130, 5, 64)])
+                                  (3, 1, 130, 5, 64), (2, 1, 200, 16, 100)])
 def test_qk_rope_cache(device, dtype, geom):
     """Bias, per-head norm and partial rotation at far positions; K and V
     land in their pages."""
