@@ -236,7 +236,8 @@ def test_kernel_groups_present(device):
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("shape", [(4, 2, 16, 8), (1, 1, 1, 1),
                                    (3, 3, 20, 36), (2, 1, 64, 70),
-                                   (2, 2, 130, 12), (6, 2, 33, 129)])
+                                   (2, 2, 130, 12), (6, 2, 33, 129),
+                                   (2, 1, 128, 64)])
 def test_delta_scan_alone(device, dtype, per_channel, shape):
     """The recurrence op, two unequal sequences in portions through slots
     that held something else, against the oracle's plain loops."""
@@ -407,7 +408,7 @@ def test_qk_rope_cache(device, dtype, geom):
     assert rel_err(gv.reshape(T, -1), wv.reshape(T, -1)) < t
 
 
-def _attend_through_cache(device, dtype, q, k, v, m, schedule, page=8):
+def _attend_through_cache(device, dtype, q, k, v, m, schedule, page=16):
     """q [T, H, dk] etc. through ops.qk_rope_cache (no norm, no rotation) and
     ops.masked_attention, fed as the schedule's portions."""
     T, H, dk = q.shape
@@ -466,6 +467,37 @@ def test_one_loud_key_at_window_and_kept_edges(device, dtype, how, loud):
     heard = want[:, 0, 0] > 5.0
     for i in range(T):
         assert bool(heard[i]) == (loud <= i and (i - loud < 37 or loud < 5))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("how", ["whole", "decoded"])
+@pytest.mark.parametrize("loud", [99, 100, 401])
+def test_loud_key_long_window_many_kept(device, dtype, how, loud):
+    """The same with a window long enough that single rows cut their keys
+    over several workgroups and with more kept keys than one key tile holds:
+    the kept keys are walked in front of the window, in whole tiles."""
+    torch.manual_seed(loud)
+    T, H, G, dk, dv = 700, 4, 1, 32, 16
+    size, first = 300, 100
+    m = {"scale": 0.5, "mask": {"size": size, "keep_first": first}}
+    q = torch.randn(T, H, dk) * 0.2
+    k = torch.randn(T, G, dk) * 0.2
+    v = torch.randn(T, G, dv)
+    q[..., 0] = 4.0
+    k[..., 0] = 0.0
+    k[loud, :, 0] = 4.0
+    v[loud] = 10.0
+    rnd = lambda t: t.to(dtype).to(F64)  # noqa: E731
+    want = orc.attend(rnd(q), rnd(k), rnd(v), m)
+    sched = [T] if how == "whole" else [405] + [1] * (T - 405)
+    got = _attend_through_cache(device, dtype, q, k, v, m, sched)
+    err = (got.to(F64) - want).abs().max()
+    assert float(err) < (2e-4 if dtype == torch.float32 else 0.15)
+    heard = want[:, 0, 0] > 5.0
+    for i in range(T):
+        assert bool(heard[i]) == (loud <= i and (i - loud < size
+                                                 or loud < first))
 
 
 @pytest.mark.parametrize("device", DEVICES)
