@@ -472,6 +472,37 @@ def test_one_loud_key_at_window_and_kept_edges(device, dtype, how, loud):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("how", ["whole", "decoded"])
+@pytest.mark.parametrize("kept", [0, 5])
+@pytest.mark.parametrize("loud", [4, 64])
+def test_loud_key_eight_heads_per_kv_head(device, dtype, how, kept, loud):
+    """Sixteen query heads on two K/V heads: single rows of such a group run
+    with the heads as matrix-core rows when no keys are kept, and on the row
+    kernel when some are."""
+    torch.manual_seed(loud + kept)
+    T, H, G, dk, dv = 150, 16, 2, 16, 8
+    m = {"scale": 0.5, "softcap": 30.0,
+         "mask": {"size": 37, "keep_first": kept}}
+    q = torch.randn(T, H, dk) * 0.2
+    k = torch.randn(T, G, dk) * 0.2
+    v = torch.randn(T, G, dv)
+    q[..., 0] = 4.0
+    k[..., 0] = 0.0
+    k[loud, :, 0] = 4.0
+    v[loud] = 10.0
+    rnd = lambda t: t.to(dtype).to(F64)  # noqa: E731
+    want = orc.attend(rnd(q), rnd(k), rnd(v), m)
+    got = _attend_through_cache(device, dtype, q, k, v, m, SCHEDULES[how])
+    err = (got.to(F64) - want).abs().max()
+    assert float(err) < (2e-4 if dtype == torch.float32 else 0.15)
+    heard = want[:, 5, 0] > 5.0
+    for i in range(T):
+        assert bool(heard[i]) == (loud <= i and (i - loud < 37
+                                                 or loud < kept))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("how", ["whole", "decoded"])
 @pytest.mark.parametrize("loud", [99, 100, 401])
 def test_loud_key_long_window_many_kept(device, dtype, how, loud):
     """The same with a window long enough that single rows cut their keys
