@@ -335,6 +335,11 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
   int lo = 0, hi = pos;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
+  // always-visible leading keys outside the window sit in front of it in a
+  // virtual key index: [wlo - nf, wlo) stands for the keys [0, nf)
+  const int wlo = lo;
+  const int vsh = lo - (ex.first > 0 ? min(ex.first, lo) : 0);
+  lo = vsh;
   if (nsplit > 1) {   // this workgroup's share of [lo, pos]; may be empty
     const int per = ((pos - lo + nsplit) / nsplit + 63) & ~63;
     lo += sp * per;
@@ -379,9 +384,10 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
   for (int kv0 = lo; kv0 <= hi; kv0 += 64) {
     __syncthreads();   // the previous tile's scores, V^T and rows are read
     if (threadIdx.x < 64) {
-      const int j = kv0 + threadIdx.x;
+      const int jv = kv0 + threadIdx.x;
+      const int j = jv < wlo ? jv - vsh : jv;
       row_lds[threadIdx.x] =
-          j <= hi ? (btr[j / page] * G + g) * page + (j % page) : -1;
+          jv <= hi ? (btr[j / page] * G + g) * page + (j % page) : -1;
     }
     __syncthreads();
     // ---- this wave's 16 keys: K fragments from the pages ----
@@ -420,14 +426,15 @@ __global__ void __launch_bounds__(256) attn_heads_mfma_kernel(
       for (int c = 0; c < DKC; ++c)
         sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             as_bf16x8(q_frag[c]), as_bf16x8(kf[c]), sa, 0, 0, 0);
-      const int j = kv0 + wid * 16 + (lane & 15);
+      const int jv = kv0 + wid * 16 + (lane & 15);
+      const int j = jv < wlo ? jv - vsh : jv;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float sv = sa[r] * scale;
         if (ex.cap > 0.f) sv = attn_softcap_fast(sv, inv_cap, ex.cap);
         if (ex.r1) sv -= attn_dist_bias(r1v[r], r2v[r], max(pos - j, 0));
         s_lds[((lane >> 4) * 4 + r) * SS + wid * 16 + (lane & 15)] =
-            (j <= hi) ? sv : AF_NEG_INF;
+            (jv <= hi) ? sv : AF_NEG_INF;
       }
     }
     __syncthreads();
@@ -575,9 +582,7 @@ AF_EXPORT int afm_attn_heads_mfma(
     int nsplit, void* part_o, void* part_ml, const void* sink, float cap,
     const void* r1, const void* r2, i64 ldv, int keep_first, void* stream) {
   if (T == 0) return 0;
-  // the head-tile kernel walks one contiguous key range: rows with
-  // always-visible leading keys go to the row kernel
-  if (keep_first > 0) return 9004;
+  if (keep_first < 0) return 9003;
   if (G <= 0 || H % G || dk < 1 || dv < 1) return 9003;
   if (ldv < dv || cap < 0.f || ((r1 == nullptr) != (r2 == nullptr))) return 9003;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
@@ -587,7 +592,7 @@ AF_EXPORT int afm_attn_heads_mfma(
                    ((uintptr_t)vc % 16 == 0);
   if (dk > 576 || dv > 512 || ((dk > 128 || dv > 128) && !vec)) return 9004;
   const AttnExtra ex{(const float*)sink, (const float*)r1, (const float*)r2,
-                     cap, ldv, 0};
+                     cap, ldv, keep_first};
   const int hpg = H / G;
   dim3 grid(T, G * ((hpg + 15) / 16), nsplit), blk(256);
   hipStream_t s = (hipStream_t)stream;

@@ -297,7 +297,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
     reach = min(x for x in (chunk, window, md.block_table.shape[1] * page)
                 if x > 0) + keep_first
     if (q.dtype == torch.bfloat16 and H // G >= HEADS_MFMA_MIN and dk <= 576
-            and dv <= 512 and keep_first == 0):
+            and dv <= 512):
         # single rows whose many heads share a K/V head: the heads are the
         # rows of the matrix-core tiles; key splits of 64-key multiples
         wgs = T * G * -(-(H // G) // 16)

@@ -476,8 +476,7 @@ def test_one_loud_key_at_window_and_kept_edges(device, dtype, how, loud):
 @pytest.mark.parametrize("loud", [4, 64])
 def test_loud_key_eight_heads_per_kv_head(device, dtype, how, kept, loud):
     """Sixteen query heads on two K/V heads: single rows of such a group run
-    with the heads as matrix-core rows when no keys are kept, and on the row
-    kernel when some are."""
+    with the heads as matrix-core rows, with and without kept keys."""
     torch.manual_seed(loud + kept)
     T, H, G, dk, dv = 150, 16, 2, 16, 8
     m = {"scale": 0.5, "softcap": 30.0,
