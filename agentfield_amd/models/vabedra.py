@@ -643,6 +643,10 @@ VABEDRA_CONFIGS = {
     # mixture (16 experts of ff 2048, top 4) matches a dense ff of 8192
     "vabedra-1b": _bench_config("vabedra-1b", 2048, 16, 16, 8, 128, 16, 4,
                                 2048),
+    # the same with 4 experts of ff 2048, all of them chosen: the parameter
+    # count of "reperax-1b"'s dense ff, no expert left idle
+    "vabedra-1b-e4": _bench_config("vabedra-1b-e4", 2048, 16, 16, 8, 128, 4,
+                                   4, 2048),
     # same width / depth / heads / vocabulary as "reperax-8b"
     "vabedra-8b": _bench_config("vabedra-8b", 4096, 32, 32, 8, 128, 16, 4,
                                 3584, vocab=128256),
